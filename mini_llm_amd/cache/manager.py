@@ -62,10 +62,11 @@ class CacheManager:
             self.last_token = torch.zeros((max_requests,), dtype=torch.int32, device=device)
 
             for gi, g in enumerate(self.groups):
-                shape = (len(g.layers), 2, self.pools[gi].num_pages, g.n_kv_heads, page_size, g.head_size)
+                planes = getattr(g, "planes", 2)
+                shape = (len(g.layers), planes, self.pools[gi].num_pages, g.n_kv_heads, page_size, g.head_size)
                 store = torch.empty(shape, dtype=dtype, device=device)
-                for li, layer in enumerate(g.layers):
-                    self.k_pages[layer], self.v_pages[layer] = store[li, 0], store[li, 1]
+                for li, layer in enumerate(g.layers):   # a group of one plane keeps no values: its rows serve as both
+                    self.k_pages[layer], self.v_pages[layer] = store[li, 0], store[li, planes - 1]
             for layer, need in self.state_needs.items():
                 self.state[layer] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
 

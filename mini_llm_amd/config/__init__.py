@@ -1,4 +1,5 @@
 from .base import ConfigError, ModelConfig, read_config_json
+from .gimozen import GimozenConfig
 from .gpt2 import GPT2Config
 from .registry import (
     Architecture,
@@ -13,6 +14,7 @@ from .registry import (
 __all__ = [
     "Architecture",
     "ConfigError",
+    "GimozenConfig",
     "GPT2Config",
     "ModelConfig",
     "architecture_name",

@@ -42,9 +42,12 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_name(raw: dict) -> str:
     names = raw.get("architectures")
-    if not isinstance(names, list) or not names or not isinstance(names[0], str):
-        raise ConfigError("config.json has no 'architectures' list naming the model class")
-    return names[0]
+    if isinstance(names, list) and names and isinstance(names[0], str):
+        return names[0]
+    name = raw.get("architecture")   # some files name their one class under this key
+    if isinstance(name, str) and name:
+        return name
+    raise ConfigError("config.json names no model class ('architectures', a list, or 'architecture')")
 
 
 def config_from_dict(raw: dict) -> ModelConfig:

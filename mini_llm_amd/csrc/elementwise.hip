@@ -11,7 +11,7 @@ template <typename T>
 __global__ void embed_kernel(int* __restrict__ tokens, const int* __restrict__ positions,
                              const int* __restrict__ sources, const int* __restrict__ token_slots,
                              const T* __restrict__ wte, const T* __restrict__ wpe,
-                             float* __restrict__ out, int width) {
+                             float* __restrict__ out, int width, float scale) {
     int row = blockIdx.x;
     int token = tokens[row];
     if (sources) {
@@ -28,17 +28,17 @@ __global__ void embed_kernel(int* __restrict__ tokens, const int* __restrict__ p
     }
     const T* token_row = wte + (size_t)token * width;
     if (wpe == nullptr) {  // positions enter the model elsewhere (or nowhere)
-        for (int i = threadIdx.x; i < width; i += blockDim.x) out_row[i] = to_float(token_row[i]);
+        for (int i = threadIdx.x; i < width; i += blockDim.x) out_row[i] = to_float(token_row[i]) * scale;
         return;
     }
     const T* position_row = wpe + (size_t)positions[row] * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x)
-        out_row[i] = to_float(token_row[i]) + to_float(position_row[i]);
+        out_row[i] = to_float(token_row[i]) * scale + to_float(position_row[i]);
 }
 
 MLLM_API int mllm_embed(int* tokens, const int* positions, const int* sources, const int* token_slots,
                         const void* wte, const void* wpe, float* out, int n_rows, int width, int table_dtype,
-                        hipStream_t stream) {
+                        float scale, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && width > 0, "embed: bad sizes rows=%d width=%d", n_rows, width);
     MLLM_REQUIRE(sources == nullptr || token_slots != nullptr, "embed: sources without token slots");
     if (n_rows == 0) return 0;
@@ -46,10 +46,10 @@ MLLM_API int mllm_embed(int* tokens, const int* positions, const int* sources, c
     mllm_count_kernel(MLLM_K_EMBED);
     if (table_dtype == MLLM_F32)
         embed_kernel<float><<<n_rows, threads, 0, stream>>>(tokens, positions, sources, token_slots, (const float*)wte,
-                                                            (const float*)wpe, out, width);
+                                                            (const float*)wpe, out, width, scale);
     else if (table_dtype == MLLM_BF16)
         embed_kernel<bf16_t><<<n_rows, threads, 0, stream>>>(tokens, positions, sources, token_slots, (const bf16_t*)wte,
-                                                             (const bf16_t*)wpe, out, width);
+                                                             (const bf16_t*)wpe, out, width, scale);
     else
         MLLM_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
     return mllm_check_launch("embed");

@@ -43,7 +43,7 @@ def cache_bytes_per_token(groups, element_size: int) -> int:
     """What one token of one request takes in the page pools: a key row and a value row in every
     cache layer. (Every group's pool holds pages for the same number of tokens; a group with a
     window gives most of them back, but is sized like the others.)"""
-    return sum(len(g.layers) * 2 * g.n_kv_heads * g.head_size * element_size for g in groups)
+    return sum(len(g.layers) * getattr(g, "planes", 2) * g.n_kv_heads * g.head_size * element_size for g in groups)
 
 
 def tokens_for_memory(groups, element_size: int, gib: float, page_size: int) -> int:

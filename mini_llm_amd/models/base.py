@@ -30,6 +30,7 @@ class CacheGroupSpec:
     n_kv_heads: int
     head_size: int
     window: int | None
+    planes: int = 2   # 1: the layers keep one row per token that serves as key and value (no value pages)
 
 
 @dataclass
@@ -86,6 +87,8 @@ class Model(Part):
         for i, block in enumerate(self.blocks):
             out[self._names["block"].format(i=i)] = block
         out[self._names["final_norm"]] = self.final_norm
+        if "head" in self._names:   # a head with a matrix of its own (a tied head has no tensors)
+            out[self._names["head"]] = self.head
         return out
 
     def canonical_tensor_name(self, name: str) -> str | None:
@@ -120,13 +123,13 @@ class Model(Part):
             need = self.blocks[call.block].mixer_part().kv_need()
             if need is None:
                 continue
-            layers = groups.setdefault((need.n_kv_heads, need.head_size, need.window), [])
+            layers = groups.setdefault((need.n_kv_heads, need.head_size, need.window, need.planes), [])
             if call.write_cache:
                 layers.append(call.cache)
             elif call.cache not in layers:
                 raise ValueError(f"a layer call reads cache layer {call.cache}, whose pages have another shape or window")
         return [
-            CacheGroupSpec(f"{'window' + str(key[2]) if key[2] else 'full'}_h{key[0]}x{key[1]}", tuple(layers), *key)
+            CacheGroupSpec(f"{'window' + str(key[2]) if key[2] else 'full'}_h{key[0]}x{key[1]}{'' if key[3] == 2 else 'p' + str(key[3])}", tuple(layers), *key)
             for key, layers in groups.items()
         ]
 

@@ -62,8 +62,8 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots=None):
-    """out[t] = wte[tokens[t]] + wpe[positions[t]] in float32 (``wpe`` None: the token row alone). A
+def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots=None, scale: float = 1.0):
+    """out[t] = scale * wte[tokens[t]] + wpe[positions[t]] in float32 (``wpe`` None: the token row alone). A
     negative token gives a zero row.
     With ``token_sources`` and ``token_slots`` the token of a row whose source is not negative is
     token_slots[source]; it is also written into ``tokens``."""
@@ -84,7 +84,7 @@ def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots
     _device_tensor(out, "out", torch.float32, 2)
     _require(tuple(out.shape) == (n, width), "out has the wrong shape")
     check(library().mllm_embed(_ptr(tokens), _ptr(positions), _ptr(token_sources), _ptr(token_slots if token_sources is not None else None),
-                               _ptr(wte), _ptr(wpe), _ptr(out), n, width, _code(wte.dtype), _stream()))
+                               _ptr(wte), _ptr(wpe), _ptr(out), n, width, _code(wte.dtype), float(scale), _stream()))
     return out
 
 
@@ -700,8 +700,24 @@ def _pending(hidden):
     return base, partials, bias, 0 if partials is None else partials.shape[0]
 
 
+@dataclass
+class NormedRows:
+    """Rows of the residual stream as a norm left them: in float32 (``stream``) and, the same numbers, in the element type
+    the next products read (``rows``; the same tensor in a 32-bit run). A layer that norms after its sums hands these on,
+    so that the next layer's products need no conversion of their own."""
+
+    stream: torch.Tensor
+    rows: torch.Tensor
+
+    @property
+    def shape(self):
+        return self.stream.shape
+
+
 def settle(hidden):
     """The stream as plain float32 rows: a tensor as it is, pending rows with their sums taken."""
+    if isinstance(hidden, NormedRows):
+        return hidden.stream
     if not isinstance(hidden, PendingRows):
         return hidden
     base, partials, bias, n_partials = _pending(hidden)
@@ -794,3 +810,155 @@ def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activa
         _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_up.data),
         _ptr(b_up), _ptr(w_down.data), _ptr(out), rows, width, inner, slice_units, EPILOGUES[activation], _stream()))
     return PendingRows(summed, out, b_down)
+
+
+# -- layers that norm after the sum, norm their heads, gate their feed-forward, or keep a latent -----------------
+def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool = False, out_dtype=None, row_index=None, with_stream: bool = False):
+    """h / sqrt(mean(h^2) + eps) * g over rows of h = alpha * x (+ addend), g = weight or, with ``one_plus``, 1 + weight.
+    x: float32 [rows, width]; addend: float32 or bfloat16 of the same shape; weight: float32 [width]. ``row_index`` (int32)
+    picks the input row of each output row. Returns the rows in ``out_dtype``, or with ``with_stream`` (the rows in float32:
+    what a residual stream goes on with, the rows in ``out_dtype``); ``out_dtype`` None: the float32 rows alone."""
+    _device_tensor(x, "x", torch.float32, 2)
+    _device_tensor(weight, "weight", torch.float32, 1)
+    width = x.shape[1]
+    _require(weight.shape[0] == width, "the gain vector does not match the row width")
+    n = x.shape[0]
+    if addend is not None:
+        _device_tensor(addend, "addend", dim=2)
+        _require(addend.shape == x.shape and row_index is None, "the addend must have the rows' shape (and rows are not gathered then)")
+    if row_index is not None:
+        _device_tensor(row_index, "row_index", torch.int32, 1)
+        n = row_index.shape[0]
+    stream = torch.empty((n, width), dtype=torch.float32, device=x.device) if with_stream or out_dtype is None else None
+    rows = torch.empty((n, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    check(library().mllm_rms_norm(_ptr(x), _ptr(addend), 0 if addend is None else _code(addend.dtype), float(alpha), _ptr(row_index), _ptr(weight),
+                                  int(bool(one_plus)), float(eps), _ptr(stream), _ptr(rows), 0 if rows is None else _code(rows.dtype), n, width, _stream()))
+    if out_dtype is None:
+        return stream
+    return (stream, rows) if with_stream else rows
+
+
+def head_norm(qkv, q_gain, k_gain, eps, positions, slots, k_pages, v_pages, n_heads, n_kv_heads, dim, vdim, *, temp_coef: float = 0.0,
+              temp_every: int = 1, write_cache: bool = True):
+    """The heads of a fused q/k/v product [rows, (n_heads + n_kv_heads) * dim + n_kv_heads * vdim]: queries RMS-normed per head
+    (gain ``q_gain`` [dim]; None: no norm) and multiplied by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1), returned as
+    [rows, n_heads * head_size]; keys normed with ``k_gain`` and values as they are stored at slots[row] of the pages
+    ([num_pages, n_kv_heads, page_size, head_size], head_size >= dim, vdim; the rest of a head is zero)."""
+    _require(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be a 2-D GPU tensor with contiguous columns")
+    num_pages, n_kv, page_size, head_size = k_pages.shape
+    _check_pages(k_pages, v_pages, n_kv_heads, head_size)
+    _require(k_pages.dtype == qkv.dtype, "pages and rows differ in element type")
+    _require(qkv.shape[1] == (n_heads + n_kv_heads) * dim + n_kv_heads * vdim, "the rows do not match the heads")
+    _require(head_size >= dim and head_size >= vdim, "the pages' heads are too small")
+    for gain, name in ((q_gain, "q_gain"), (k_gain, "k_gain")):
+        if gain is not None:
+            _device_tensor(gain, name, torch.float32, 1)
+            _require(gain.shape[0] == dim, f"{name} does not match the heads")
+    n = qkv.shape[0]
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _device_tensor(slots, "slots", torch.int32, 1)
+    _require(positions.shape[0] >= n and slots.shape[0] >= n, "fewer positions or slots than rows")
+    q = torch.empty((n, n_heads * head_size), dtype=qkv.dtype, device=qkv.device)
+    check(library().mllm_head_norm(_ptr(qkv), qkv.stride(0), _ptr(q_gain), _ptr(k_gain), float(eps), float(temp_coef), int(temp_every), _ptr(positions),
+                                   _ptr(slots), _ptr(q), _ptr(k_pages), _ptr(v_pages), n, n_heads, n_kv_heads, dim, vdim, head_size, page_size,
+                                   int(bool(write_cache)), _code(qkv.dtype), _stream()))
+    return q
+
+
+def silu_mul(both):
+    """silu(a) * b for rows [a | b] of a fused gate / up product: [rows, 2 * inner] -> [rows, inner]."""
+    _device_tensor(both, "both", dim=2)
+    _require(both.shape[1] % 2 == 0, "the rows do not hold two halves")
+    n, inner = both.shape[0], both.shape[1] // 2
+    out = torch.empty((n, inner), dtype=both.dtype, device=both.device)
+    check(library().mllm_silu_mul(_ptr(both), _ptr(out), n, inner, _code(both.dtype), _stream()))
+    return out
+
+
+def latent_rows(q, dkv, gain, eps, frequencies, magnitude, rot_dims, positions, slots, pages, n_heads, dim, rot, rank):
+    """A latent-attention layer's row-wise work. q: [rows, n_heads * (dim + rot)]; dkv: [rows, rank + rot] or None (the layer
+    reads rows another layer keeps). Returns q_full, float32 [rows, n_heads, row_size] with the rotated query part at
+    [rank, rank + rot) and zeros behind (the first ``rank`` elements are left for ``heads_linear``); stores, with dkv, the
+    RMS-normed latent (gain [rank]) and the rotated key part at slots[row] of pages [num_pages, 1, page_size, row_size].
+    ``frequencies``: float32 [rot_dims / 2], the angle per position of each rotated pair; ``magnitude`` multiplies cos and sin."""
+    _require(q.is_cuda and q.dim() == 2 and q.stride(1) == 1, "q must be a 2-D GPU tensor with contiguous columns")
+    _device_tensor(pages, "pages", q.dtype, 4)
+    _require(pages.shape[1] == 1, "a latent cache has one row per token")
+    page_size, row_size = pages.shape[2], pages.shape[3]
+    n = q.shape[0]
+    _require(q.shape[1] == n_heads * (dim + rot) and row_size >= rank + rot, "the rows do not match the heads")
+    if dkv is not None:
+        _require(dkv.is_cuda and dkv.dim() == 2 and dkv.stride(1) == 1 and dkv.dtype == q.dtype and tuple(dkv.shape) == (n, rank + rot), "dkv does not match the latent")
+        _device_tensor(gain, "gain", torch.float32, 1)
+        _require(gain.shape[0] == rank, "the gain vector does not match the latent")
+    _device_tensor(frequencies, "frequencies", torch.float32, 1)
+    _require(rot_dims % 2 == 0 and rot_dims <= rot and frequencies.shape[0] >= rot_dims // 2, "the rotation does not fit the rotated part")
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _device_tensor(slots, "slots", torch.int32, 1)
+    _require(positions.shape[0] >= n and slots.shape[0] >= n, "fewer positions or slots than rows")
+    q_full = torch.empty((n, n_heads, row_size), dtype=torch.float32, device=q.device)
+    check(library().mllm_latent_rows(_ptr(q), q.stride(0), _ptr(dkv), 0 if dkv is None else dkv.stride(0), _ptr(gain if dkv is not None else None), float(eps),
+                                     _ptr(frequencies), float(magnitude), int(rot_dims), _ptr(positions), _ptr(slots), _ptr(q_full), _ptr(pages), n, n_heads,
+                                     dim, rot, rank, row_size, page_size, _code(q.dtype), _stream()))
+    return q_full
+
+
+def heads_linear(x, weight, out, *, n_heads, k, x_head_stride, n_out=None, gate=None):
+    """out[row, h, :n] = x[row, h, :k] @ weight[h].T (* sigmoid(gate[row, h, :n])): one small product per head. x: 2-D or 3-D,
+    its rows ``x.stride(0)`` apart and its heads ``x_head_stride``; weight: [n_heads, n, k]; out: [rows, n_heads, >= n] (a view
+    whose last elements may belong to someone else); gate: [rows, n_heads * n]."""
+    _require(x.is_cuda and x.stride(-1) == 1, "x must be on the GPU with contiguous elements")
+    _device_tensor(weight, "weight", dim=3)
+    _require(weight.shape[0] == n_heads and weight.shape[2] == k, "weight does not match the heads")
+    n = weight.shape[1] if n_out is None else n_out
+    _require(out.is_cuda and out.dim() == 3 and out.shape[1] == n_heads and out.shape[2] >= n and out.stride(2) == 1, "out must be [rows, heads, >= n]")
+    rows = x.shape[0]
+    _require(out.shape[0] == rows, "x and out differ in rows")
+    _require(x.stride(0) >= (n_heads - 1) * x_head_stride + k, "x's rows are too short for the heads")
+    if gate is not None:
+        _require(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and tuple(gate.shape) == (rows, n_heads * n), "the gate does not match the output")
+    check(library().mllm_heads_linear(_ptr(x), _code(x.dtype), x.stride(0), int(x_head_stride), _ptr(weight), _code(weight.dtype), _ptr(gate),
+                                      0 if gate is None else _code(gate.dtype), 0 if gate is None else gate.stride(0), _ptr(out), _code(out.dtype), out.stride(0), out.stride(1), rows, n_heads,
+                                      n, k, _stream()))
+    return out
+
+
+LATENT_RUN_MIN = 256   # cached rows a run of a token's keys should at least hold
+
+
+def latent_attention_supported(rank: int, row_size: int, dtype) -> bool:
+    return bool(library().mllm_latent_attention_supported(int(rank), int(row_size), _code(dtype)))
+
+
+def latent_attention(q_full, pages, sinks, token_request, positions, block_tables, rank, scale, max_len=None):
+    """Causal attention of each row's heads over its request's cached rows: score = scale * q_full[row, h] . cached row, softmax
+    with exp(sinks[h]) in the denominator (``sinks`` None: without), the sum taken over the rows' first ``rank`` elements.
+    q_full: float32 [rows, n_heads, row_size]; pages [num_pages, 1, page_size, row_size]. Returns float32 [rows, n_heads,
+    rank]. Few rows with many keys are cut into runs of keys, a block each (``max_len``: the longest sequence of the batch)."""
+    _device_tensor(q_full, "q_full", torch.float32, 3)
+    _device_tensor(pages, "pages", dim=4)
+    n, n_heads, row_size = q_full.shape
+    _require(pages.shape[1] == 1 and pages.shape[3] == row_size, "pages and queries differ in row size")
+    page_size = pages.shape[2]
+    if sinks is not None:
+        _device_tensor(sinks, "sinks", torch.float32, 1)
+        _require(sinks.shape[0] == n_heads, "one sink per head")
+    _device_tensor(token_request, "token_request", torch.int32, 1)
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _device_tensor(block_tables, "block_tables", torch.int32, 2)
+    _require(token_request.shape[0] >= n and positions.shape[0] >= n, "fewer positions than rows")
+    out = torch.empty((n, n_heads, rank), dtype=torch.float32, device=q_full.device)
+    if n == 0:
+        return out
+    reach = block_tables.shape[1] * page_size
+    longest = reach if max_len is None else max(1, min(int(max_len), reach))
+    n_runs, units = 1, _compute_units(q_full.device)
+    groups = n * -(-n_heads // 16)
+    while 2 * groups * n_runs <= 2 * units and 2 * n_runs * LATENT_RUN_MIN <= longest:
+        n_runs *= 2
+    run_length = -(-reach // n_runs) if n_runs > 1 else reach
+    parts = torch.empty((n, n_heads, n_runs, rank + 2), dtype=torch.float32, device=q_full.device) if n_runs > 1 else None
+    check(library().mllm_latent_attention(_ptr(q_full), _ptr(pages), _ptr(sinks), _ptr(out), _ptr(parts), _ptr(token_request), _ptr(positions),
+                                          _ptr(block_tables), block_tables.shape[1], n, n_heads, int(rank), row_size, page_size, float(scale),
+                                          n_runs, run_length, _code(pages.dtype), _stream()))
+    return out

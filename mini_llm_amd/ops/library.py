@@ -15,7 +15,7 @@ _library: ctypes.CDLL | None = None
 
 P = c_void_p
 _SIGNATURES = {
-    "mllm_embed": [P, P, P, P, P, P, P, c_int, c_int, c_int, P],
+    "mllm_embed": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_float, P],
     "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
     "mllm_add": [P, P, P, c_longlong, c_int, P],
     "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
@@ -47,6 +47,13 @@ _SIGNATURES = {
     "mllm_linear_split_static": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_static_scratch_prepare": [],
     "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
+    "mllm_rms_norm": [P, P, c_int, c_float, P, P, c_int, c_float, P, P, c_int, c_int, c_int, P],
+    "mllm_head_norm": [P, c_int, P, P, c_float, c_float, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_latent_rows": [P, c_int, P, c_int, P, c_float, P, c_float, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_silu_mul": [P, P, c_int, c_int, c_int, P],
+    "mllm_heads_linear": [P, c_int, c_int, c_int, P, c_int, P, c_int, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_latent_attention_supported": [c_int, c_int, c_int],
+    "mllm_latent_attention": [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
 }
 
 

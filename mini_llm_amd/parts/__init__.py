@@ -1,19 +1,21 @@
-from .attention import CausalSelfAttention
+from .attention import CausalSelfAttention, NormedHeadAttention
 from .base import (
     BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS,
     Block, FeedForward, KVNeed, LayerContext, Mixer, Norm, Part, PositionEncoding, StateNeed,
     make_part, register_part,
 )
-from .block import PreNormBlock
-from .embedding import TiedHead, TokenEmbedding
-from .feedforward import DenseMLP
+from .block import PostNormBlock, PreNormBlock
+from .embedding import LinearHead, TiedHead, TokenEmbedding
+from .feedforward import DenseMLP, GatedMLP
+from .latent_attention import LatentAttention
 from .linear import Linear
-from .norms import LayerNorm
-from .positions import LearnedPositions
+from .norms import LayerNorm, RMSNorm
+from .positions import LearnedPositions, RotaryEncoding
 
 __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS",
     "Block", "FeedForward", "KVNeed", "LayerContext", "Mixer", "Norm", "Part", "PositionEncoding", "StateNeed",
     "make_part", "register_part",
     "CausalSelfAttention", "PreNormBlock", "TiedHead", "TokenEmbedding", "DenseMLP", "Linear", "LayerNorm", "LearnedPositions",
+    "NormedHeadAttention", "LatentAttention", "PostNormBlock", "LinearHead", "GatedMLP", "RMSNorm", "RotaryEncoding",
 ]

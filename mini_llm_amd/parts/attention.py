@@ -100,4 +100,74 @@ class CausalSelfAttention(Mixer):
         return self.forward(x, hidden, ctx)
 
 
+class NormedHeadAttention(Mixer):
+    """Causal attention with grouped key/value heads, separate q / k / v / o matrices without biases (stored [out, in] under
+    their bare names), an RMS norm over each query and key head (one gain vector of ``dim`` for all heads, eps ``eps``), no
+    rotation, a temperature on the queries that grows with the position, 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1),
+    a given score ``scale`` and an ordinary softmax. Query/key heads have ``dim`` elements and value heads ``vdim``.
+
+    q, k and v run as one product over the three matrices laid behind each other; one kernel norms the heads, applies the
+    temperature and stores keys and values in their pages. The pages hold heads of ``head_size`` = the larger of dim and vdim
+    (rounded up to a multiple of 16), zeros beyond a head's own elements, so that the paged attention kernels of equal key
+    and value sizes serve; the output matrix gets zero columns to match."""
+
+    graph_safe = True
+    short_portion = kernels.DECODE_MAX_Q_LEN
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: float, eps: float, temp_coef: float = 0.0,
+                 temp_every: int = 1, window: int | None = None, qk_norm: bool = True):
+        if n_heads < 1 or n_kv_heads < 1 or n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} key/value heads")
+        self.head_size = -(-max(dim, vdim) // 16) * 16
+        if not 1 <= self.head_size <= MAX_HEAD_SIZE:
+            raise ValueError(f"heads of {max(dim, vdim)} are wider than the attention kernels take ({MAX_HEAD_SIZE})")
+        if temp_every < 1:
+            raise ValueError(f"the temperature's period must be at least 1, not {temp_every}")
+        self.width, self.n_heads, self.n_kv_heads, self.dim, self.vdim = width, n_heads, n_kv_heads, dim, vdim
+        self.scale, self.eps, self.temp_coef, self.temp_every, self.window, self.qk_norm = float(scale), float(eps), float(temp_coef), int(temp_every), window, qk_norm
+        self.qkv = self.o = self.q_norm = self.k_norm = None
+
+    def tensor_specs(self):
+        from ..weights.spec import TABLE, VECTOR, Normal, TensorSpec
+
+        std = self.width ** -0.5
+        specs = {"q": TensorSpec((self.n_heads * self.dim, self.width), TABLE, Normal(std)),
+                 "k": TensorSpec((self.n_kv_heads * self.dim, self.width), TABLE, Normal(std)),
+                 "v": TensorSpec((self.n_kv_heads * self.vdim, self.width), TABLE, Normal(std)),
+                 "o": TensorSpec((self.width, self.n_heads * self.vdim), TABLE, Normal((self.n_heads * self.vdim) ** -0.5))}
+        if self.qk_norm:
+            specs["q.norm"] = TensorSpec((self.dim,), VECTOR, Normal(0.1, mean=1.0))
+            specs["k.norm"] = TensorSpec((self.dim,), VECTOR, Normal(0.1, mean=1.0))
+        return specs
+
+    def bind(self, tensors):
+        q, k, v, o = tensors["q"], tensors["k"], tensors["v"], tensors["o"]
+        self.q_norm, self.k_norm = tensors.get("q.norm"), tensors.get("k.norm")
+        if self.head_size != self.vdim:   # the attention leaves heads of head_size: the columns beyond a head's vdim meet zeros
+            wide = torch.zeros((self.width, self.n_heads, self.head_size), dtype=o.dtype, device=o.device)
+            wide[:, :, : self.vdim] = o.view(self.width, self.n_heads, self.vdim)
+            o = wide.view(self.width, self.n_heads * self.head_size)
+        fused = torch.cat([q, k, v], dim=0).contiguous()
+        self.qkv, self.o = (kernels.pack_matrix(fused), kernels.pack_matrix(o.contiguous())) if fused.is_cuda else (fused, o)
+
+    def kv_need(self):
+        return KVNeed(self.n_kv_heads, self.head_size, self.window)
+
+    def forward(self, x, residual, ctx: LayerContext):
+        """The branch alone (float32) when ``residual`` is None, else residual + branch."""
+        batch = ctx.batch
+        q = kernels.head_norm(kernels.linear(x, self.qkv), self.q_norm, self.k_norm, self.eps, batch.positions, ctx.group.slots, ctx.k_pages,
+                              ctx.v_pages, self.n_heads, self.n_kv_heads, self.dim, self.vdim, temp_coef=self.temp_coef,
+                              temp_every=self.temp_every, write_cache=ctx.write_cache)
+        mixed = kernels.paged_attention(
+            q, ctx.k_pages, ctx.v_pages, batch.token_request, batch.positions, ctx.group.block_tables,
+            self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
+            max_q_len=batch.max_q_len, max_len=batch.max_total_len, q_starts=batch.q_starts, context_lens=batch.context_lens,
+            first_row=getattr(batch, "first_row", 0),
+            **({"short_rows": batch.short_rows, "short_requests": batch.short_requests} if batch.short_portion <= kernels.DECODE_MAX_Q_LEN else {}),
+        )
+        return kernels.linear(mixed, self.o, residual=residual, out_dtype=torch.float32)
+
+
 register_part("mixer", "causal_attention", CausalSelfAttention)
+register_part("mixer", "normed_head_attention", NormedHeadAttention)

@@ -30,7 +30,7 @@ class Part:
     def bind(self, tensors: dict) -> None:
         """Receives this part's own tensors, already on the device in the kept layout."""
         for name, tensor in tensors.items():
-            setattr(self, name.replace(".", "_"), tensor)
+            setattr(self, name.replace(".", "_") or "weight", tensor)   # a part's one tensor may carry the part's own name (local name "")
 
     # -- walking the tree ------------------------------------------------------------------
     def named_tensor_specs(self, prefix: str = "") -> dict[str, TensorSpec]:
@@ -59,6 +59,7 @@ class KVNeed:
     n_kv_heads: int
     head_size: int
     window: int | None = None
+    planes: int = 2   # 2: keys and values; 1: one row per token that serves as both (a latent cache): no value pages are kept
 
 
 @dataclass(frozen=True)

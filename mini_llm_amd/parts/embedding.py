@@ -3,17 +3,24 @@
 from __future__ import annotations
 
 from ..ops import kernels
-from ..weights.spec import TABLE, Normal, TensorSpec
+from ..weights.spec import MATRIX, TABLE, Normal, TensorSpec
 from .base import Part, PositionEncoding
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab_size: int, width: int):
-        self.vocab_size, self.width = vocab_size, width
+    """``scale`` multiplies the token rows (in 32-bit, as they are gathered). ``tensor_name``: the table's name behind the
+    part's prefix ("" where the part's own name is the tensor's)."""
+
+    def __init__(self, vocab_size: int, width: int, scale: float = 1.0, tensor_name: str = "weight", std: float = 0.02):
+        self.vocab_size, self.width, self.scale = vocab_size, width, float(scale)
+        self._tensor_name, self._std = tensor_name, std
         self.weight = None
 
     def tensor_specs(self):
-        return {"weight": TensorSpec((self.vocab_size, self.width), TABLE, Normal(0.02))}
+        return {self._tensor_name: TensorSpec((self.vocab_size, self.width), TABLE, Normal(self._std))}
+
+    def bind(self, tensors):
+        self.weight = tensors[self._tensor_name]
 
     def forward(self, tokens, positions, position_encoding: PositionEncoding | None, token_sources=None, token_slots=None):
         """[rows, width] float32: token rows, with the position rows added when the encoding
@@ -22,7 +29,7 @@ class TokenEmbedding(Part):
         ``token_slots``: rows whose token is still on the device, in the slot the sampler left it
         in (kernels.embed)."""
         table = position_encoding.weight if position_encoding is not None and position_encoding.stage == "embedding" else None
-        return kernels.embed(tokens, positions, self.weight, table, token_sources=token_sources, token_slots=token_slots)
+        return kernels.embed(tokens, positions, self.weight, table, token_sources=token_sources, token_slots=token_slots, scale=self.scale)
 
 
 class TiedHead(Part):
@@ -44,3 +51,29 @@ class TiedHead(Part):
         if not kernels.best_per_row(x.shape[0], self.embedding.weight, x.dtype):
             return None
         return kernels.linear_best(x, self.embedding.weight)
+
+
+class LinearHead(Part):
+    """logits = x . W^T with a matrix of its own, [vocab, width], no bias."""
+
+    def __init__(self, vocab_size: int, width: int, tensor_name: str = "weight"):
+        self.vocab_size, self.width = vocab_size, width
+        self._tensor_name = tensor_name
+        self.weight = None
+
+    def tensor_specs(self):
+        return {self._tensor_name: TensorSpec((self.vocab_size, self.width), MATRIX, Normal(self.width ** -0.5))}
+
+    def bind(self, tensors):
+        self.weight = tensors[self._tensor_name]
+
+    def forward(self, x):
+        import torch
+
+        return kernels.linear(x, self.weight, out_dtype=torch.float32)
+
+    def forward_best(self, x):
+        """See TiedHead.forward_best."""
+        if not kernels.best_per_row(x.shape[0], self.weight, x.dtype):
+            return None
+        return kernels.linear_best(x, self.weight)

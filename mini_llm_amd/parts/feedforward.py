@@ -47,4 +47,33 @@ class DenseMLP(FeedForward):
         return self.down.forward_pending(self.up.forward(x, activation=self.activation, packed_out=packed_out), hidden)
 
 
+class GatedMLP(FeedForward):
+    """down(silu(gate x) * (up x)), no biases; the three matrices are stored [out, in] under their bare names. Gate and up run
+    as one product over the two matrices laid behind each other, the activation and the multiplication as one kernel over its
+    halves, and the residual sum (if a residual is given) inside the down product."""
+
+    def __init__(self, width: int, inner: int, names=("gate", "up", "down")):
+        self.width, self.inner = width, inner
+        self._names = names
+        self.gate_up = self.down = None
+
+    def tensor_specs(self):
+        from ..weights.spec import MATRIX, TABLE, Normal, TensorSpec
+
+        gate, up, down = self._names
+        return {gate: TensorSpec((self.inner, self.width), TABLE, Normal(self.width ** -0.5)),
+                up: TensorSpec((self.inner, self.width), TABLE, Normal(self.width ** -0.5)),
+                down: TensorSpec((self.width, self.inner), MATRIX, Normal(self.inner ** -0.5))}
+
+    def bind(self, tensors):
+        gate, up, down = (tensors[name] for name in self._names)
+        self.gate_up = kernels.pack_matrix(torch.cat([gate, up], dim=0).contiguous()) if gate.is_cuda else torch.cat([gate, up], dim=0)
+        self.down = down
+
+    def forward(self, x, residual):
+        inner = kernels.silu_mul(kernels.linear(x, self.gate_up))
+        return kernels.linear(inner, self.down, residual=residual, out_dtype=torch.float32)
+
+
 register_part("feed_forward", "dense_mlp", DenseMLP)
+register_part("feed_forward", "gated_mlp", GatedMLP)

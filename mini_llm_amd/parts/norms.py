@@ -32,4 +32,35 @@ class LayerNorm(Norm):
         return kernels.layernorm(hidden, self.weight, self.bias, self.eps, out_dtype=out_dtype, with_sums=True, packed_out=packed)
 
 
+class RMSNorm(Norm):
+    """x / sqrt(mean(x^2) + eps) * g, in 32-bit. ``one_plus``: the stored vector lies around zero and g = 1 + weight.
+    ``tensor_name``: the vector's name behind the part's prefix ("" where the part's own name is the tensor's)."""
+
+    def __init__(self, width: int, eps: float, one_plus: bool = False, tensor_name: str = "weight"):
+        if not eps > 0:
+            raise ValueError(f"eps must be positive, not {eps}")
+        self.width, self.eps, self.one_plus = width, float(eps), bool(one_plus)
+        self._tensor_name = tensor_name
+        self.weight = None
+
+    def tensor_specs(self):
+        return {self._tensor_name: TensorSpec((self.width,), VECTOR, Normal(0.05, mean=0.0 if self.one_plus else 1.0))}
+
+    def bind(self, tensors):
+        self.weight = tensors[self._tensor_name]
+
+    def forward(self, x, out_dtype, row_index=None):
+        return kernels.rms_norm(x, self.weight, self.eps, one_plus=self.one_plus, out_dtype=out_dtype, row_index=row_index)
+
+    def forward_sum(self, x, addend, alpha, out_dtype):
+        """norm(alpha * x + addend) -> kernels.NormedRows: the rows in float32 and in ``out_dtype``, from one kernel (a layer
+        that norms after its sums goes on with both)."""
+        if out_dtype == x.dtype:
+            stream = kernels.rms_norm(x, self.weight, self.eps, addend=addend, alpha=alpha, one_plus=self.one_plus)
+            return kernels.NormedRows(stream, stream)
+        return kernels.NormedRows(*kernels.rms_norm(x, self.weight, self.eps, addend=addend, alpha=alpha, one_plus=self.one_plus,
+                                                    out_dtype=out_dtype, with_stream=True))
+
+
 register_part("norm", "layernorm", LayerNorm)
+register_part("norm", "rmsnorm", RMSNorm)

@@ -21,4 +21,49 @@ class LearnedPositions(PositionEncoding):
         return self.n_positions
 
 
+class RotaryEncoding(PositionEncoding):
+    """Rotation of the first ``dims`` elements of a head by an angle that grows with the position, element i paired with
+    element i + dims / 2 ("rotate half"): pair i turns by p * f_i with f_i = base^(-2i / dims). It has no tensors; the mixer
+    that holds it applies it to its queries and keys (``stage`` "mixer") with ``frequencies`` and ``magnitude``.
+
+    ``scaling`` = {factor, original, fast, slow} stretches the slow pairs for sequences longer than ``original`` positions
+    (YaRN: Peng, Quesnelle, Fan, Shippole, "YaRN: Efficient Context Window Extension of Large Language Models"): with
+    pair(t) = dims * ln(original / (2 pi t)) / (2 ln base), the pair that turns t times within the original length, lo =
+    max(floor(pair(fast)), 0), hi = min(ceil(pair(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+    the frequency becomes f_i / factor * ramp_i + f_i * (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+
+    stage = "mixer"
+
+    def __init__(self, dims: int, base: float, scaling: dict | None = None):
+        import math
+
+        if dims < 0 or dims % 2:
+            raise ValueError(f"a rotation pairs elements: {dims} is not an even number of them")
+        if not base > 0:
+            raise ValueError(f"the base must be positive, not {base}")
+        self.dims, self.base, self.scaling = dims, float(base), dict(scaling) if scaling else None
+        values = [self.base ** (-2.0 * i / dims) for i in range(dims // 2)]
+        self.magnitude = 1.0
+        if self.scaling:
+            factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+            pair = lambda turns: dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+            lo = max(math.floor(pair(float(self.scaling["fast"]))), 0)
+            hi = min(math.ceil(pair(float(self.scaling["slow"]))), dims - 1)
+            for i, f in enumerate(values):
+                ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+                values[i] = f / factor * ramp + f * (1.0 - ramp)
+            self.magnitude = 0.1 * math.log(factor) + 1.0
+        self.values = values   # float64 on the host; ``frequencies`` rounds them to 32-bit on the device
+        self._on_device = {}
+
+    def frequencies(self, device):
+        import torch
+
+        key = str(device)
+        if key not in self._on_device:
+            self._on_device[key] = torch.tensor(self.values or [0.0], dtype=torch.float64).to(torch.float32).to(device)
+        return self._on_device[key]
+
+
 register_part("position_encoding", "learned", LearnedPositions)
+register_part("position_encoding", "rotary", RotaryEncoding)
