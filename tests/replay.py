@@ -38,7 +38,8 @@ def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page_size=None, time
     done = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=timeout)
     assert done.returncode == 0, f"trace_run failed ({done.returncode}):\n{done.stderr[-3000:]}"
     assert [l for l in done.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
-    vocab = json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"]
+    config = json.loads((Path(model_dir) / "config.json").read_text())
+    vocab = config["vocab_size"] if "vocab_size" in config else config["vocab"]
     out = {}
     for s in steps:
         wanted = sum(len(e.get("want", [])) for e in s["entries"])
