@@ -81,7 +81,7 @@ def test_head_norm_writes_queries_keys_and_values(dtype, dim, vdim, heads, kv_he
     q = k.head_norm(gpu(qkv, dtype), gpu(qg), gpu(kg), eps, torch.tensor(positions, dtype=torch.int32).cuda(), torch.tensor(slots, dtype=torch.int32).cuda(),
                     k_pages, v_pages, heads, kv_heads, dim, vdim, temp_coef=0.3, temp_every=7)
     temp = plain.query_temperature(positions, 0.3, 7)
-    assert temp[4] > temp[3] == 1.0 and temp[7] > temp[6] > temp[5]   # the steps lie where floor((p + 1) / 7) changes
+    assert temp[2] == 1.0 < temp[3] == temp[4] == temp[5] < temp[6] == temp[7]   # the steps lie where floor((p + 1) / 7) changes: at 6 and at 13
     want_q = plain.rms_norm(qkv[:, : heads * dim].reshape(rows, heads, dim), qg, eps) * temp[:, None, None]
     got_q = q.float().cpu().numpy().reshape(rows, heads, head_size)
     np.testing.assert_allclose(got_q[:, :, :dim], want_q, **tol(dtype))
