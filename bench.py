@@ -329,6 +329,136 @@ def _by_entry_point(names, each):
     return table
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# --design gimozen: the Gimozen design beside GPT-2 at equal sizes
+# ---------------------------------------------------------------------------------------------------------------------
+DESIGN_SIZES = {   # width, layers; heads of 64; GPT-2's inner size 4 x width, the gated feed-forward's 8/3 x width (equal weights)
+    "small": (768, 12),
+    "medium": (1024, 24),
+}
+_KERNEL_CLASSES = {
+    "products": ("gemm", "gemm_split", "gemm_qkv_cache", "gemm_best", "heads_linear"),
+    "attention": ("attention", "attention_decode", "attention_prefill", "latent_attention"),
+    "row-wise": ("layernorm", "pending_layernorm", "rms_norm", "head_norm", "latent_rows", "silu_mul", "pending_sum", "add", "cache_write", "embed"),
+    "layer kernels": ("decode_attention_half", "decode_mlp_half"),
+    "choice": ("choose", "sample"),
+}
+
+
+def gimozen_shape(width: int, layers: int, vocab: int = 50257) -> dict:
+    """Layers of normed-head attention (heads of 64, as many key/value heads) with every fourth a latent layer (a latent of
+    256 and a rotated part of 32 for heads of 64 + 32: a cached row of 288 elements against the 2 x width of an attention
+    layer), of which every second borrows the rows of the one before it; feed-forwards of 8/3 x width."""
+    heads = width // 64
+    ff = -(-(8 * width // 3) // 64) * 64
+    rot = {"dims": 32, "base": 10000.0, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}
+    out, latent_at = [], None
+    for index in range(layers):
+        if index % 4 == 2:
+            mixer = {"heads": heads, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": 256, "rot": rot, "scale": 96 ** -0.5}
+            if latent_at is not None:
+                mixer["kv_from"], latent_at = latent_at, None
+            else:
+                latent_at = index
+            out.append({"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+        else:
+            out.append({"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+                        "mixer": {"heads": heads, "kv_heads": heads, "dim": 64, "vdim": 64, "scale": 0.125, "q_temp": {"coef": 0.1, "every": 256}}})
+    return {"architecture": "Gimozen", "vocab": vocab, "width": width, "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-5},
+            "postln_alpha": 1.0, "layers": out}
+
+
+def measure_design(args) -> dict:
+    """Prefill and decode throughput of the Gimozen design and of GPT-2 with as many layers of the same width (random
+    weights), and where each model's step spends its time, by class of kernel, inside a prompt step and a decode step."""
+    import numpy as np
+    import torch
+
+    from mini_llm_amd.config import config_from_dict
+    from mini_llm_amd.engine import StepEntry
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    width, layers = DESIGN_SIZES[args.shape]
+    raws = {"gimozen": gimozen_shape(width, layers),
+            "gpt2": {"architectures": ["GPT2LMHeadModel"], "n_layer": layers, "n_embd": width, "n_head": width // 64, "n_inner": 4 * width,
+                     "vocab_size": 50257, "n_positions": CONTEXT, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}}
+    record = {"design": "gimozen beside gpt2", "width": width, "layers": layers, "dtype": args.dtype, "context": CONTEXT, "prompt_len": args.prompt_len}
+    rng = np.random.default_rng(SEED + 7)
+    for name, raw in raws.items():
+        config = config_from_dict(raw)
+        engine = Engine.from_random(config, SEED, EngineOptions(dtype=args.dtype, max_sessions=64, max_tokens=64 * CONTEXT, max_length=CONTEXT))
+        figures = {}
+        for batch, steps in ((1, 64), (8, 128), (64, 64)):
+            seconds, _ = _DesignDecode(engine, batch, args.prompt_len).run(steps, 8)
+            figures[f"decode_b{batch}_tokens_per_s"] = round(batch * steps / seconds, 1)
+            figures[f"decode_b{batch}_ms_per_step"] = round(seconds / steps * 1e3, 4)
+        prompts = [rng.integers(0, config.vocab_size, CONTEXT).astype(np.int32) for _ in range(2)]
+        times = []
+        for _ in range(4 + 2 + engine.runner.portion_graph_after):
+            handles = [engine.try_take_cache() for _ in prompts]
+            torch.cuda.synchronize()
+            begin = time.perf_counter()
+            engine.runner.step([StepEntry(h, p, [len(p) - 1]) for h, p in zip(handles, prompts)])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - begin)
+            for h in handles:
+                engine.release_cache(h)
+        seconds = float(np.median(times[-4:]))
+        figures["prefill_tokens_per_s"], figures["prefill_ms"] = round(2 * CONTEXT / seconds, 1), round(seconds * 1e3, 3)
+        if not args.no_kernels:
+            def prompt_step():
+                handles = [engine.try_take_cache() for _ in prompts]
+                return [StepEntry(h, p, [len(p) - 1]) for h, p in zip(handles, prompts)], handles
+
+            context = (3 * CONTEXT // 4) // 64 * 64 + 8
+            stored = [rng.integers(0, config.vocab_size, context).tolist() for _ in range(8)]
+
+            def decode_step():
+                handles = [engine.try_take_cache() for _ in range(8)]
+                for i in range(0, 8, 4):
+                    engine.runner.step([StepEntry(h, tokens, []) for h, tokens in zip(handles[i : i + 4], stored[i : i + 4])])
+                return [StepEntry(h, [int(rng.integers(0, config.vocab_size))], [0]) for h in handles], handles
+
+            for what, make, choose in (("prefill_step", prompt_step, False), ("decode_step_b8", decode_step, True)):
+                names, each = kernel_times_inside_a_step(engine, make, choose=choose, reps=3)
+                table = _by_entry_point(names, each)
+                classes = {}
+                for kind, members in _KERNEL_CLASSES.items():
+                    found = [table[m] for m in members if m in table]
+                    if found:
+                        classes[kind] = {"launches": sum(f[0] for f in found), "us": round(sum(f[1] for f in found), 1)}
+                figures[what] = {"us": round(sum(each), 1), "kernels": len(names), "by_class": classes, "by_entry_point": table}
+        record[name] = figures
+        engine.close()
+        del engine
+        torch.cuda.empty_cache()
+    return record
+
+
+class _DesignDecode(DecodeBench):
+    """DecodeBench without the bytes of a GPT-2 step (its roofline is priced from the kernels' own bytes instead)."""
+
+    def run(self, steps: int, warmup: int):
+        import torch
+
+        self.start()
+        for _ in range(warmup):
+            self.last = self.engine.decode_batch(self.handles, self.last)
+            self.length += 1
+        assert self.length + steps < CONTEXT, "the timed steps must fit the context"
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        self.engine.decode_batch_enqueue(self.handles)
+        for _ in range(steps - 1):
+            self.engine.decode_batch_enqueue(self.handles)
+            self.last = self.engine.take()
+        self.last = self.engine.take()
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - begin
+        self.stop()
+        return seconds, 0.0
+
+
 def check_before_timing(engine, host_weights=None, n_new: int = 8):
     """The gate before anything is timed, as the reference's bench has one (engine/bench/bench.c:30-31,
     92-113: its GPU against its CPU path on 8 tokens, scaled difference <= 1e-3 and the same next
@@ -511,6 +641,8 @@ def main() -> int:
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
     parser.add_argument("--step-by-step", action="store_true", help="--serving reads every step's tokens before it launches the next")
+    parser.add_argument("--design", default=None, choices=("gimozen",), help="the Gimozen design beside GPT-2 with as many layers of the same width (--shape small|medium): "
+                        "prefill and decode throughput of both, and where their steps spend the time")
     parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -523,6 +655,12 @@ def main() -> int:
 
     if args.serving:
         emit({"serving": measure_serving(args.dtype, args.temperature, not args.step_by_step)}, args.json)
+        return 0
+
+    if args.design:
+        if args.shape not in DESIGN_SIZES:
+            parser.error(f"--design runs --shape {' or '.join(DESIGN_SIZES)}")
+        emit(measure_design(args), args.json)
         return 0
 
     from mini_llm_amd.config import config_from_dict
