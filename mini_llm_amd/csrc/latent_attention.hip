@@ -4,7 +4,7 @@
 // A head's key is W_uk c (+ the shared rotated part) and its value W_uv c. Neither is ever formed: the key expansion is folded
 // into the query, q' = W_uk^T q, so that a score is q' . c + q_rot . k_rot, a dot product with the cached row as it lies; the
 // weighted sum is taken over the latents, o' = sum_j p_j c_j, and expanded once per query, o = W_uv o'. All heads of a token
-// read the same rows, so a block takes a token and a wave a head, and a tile of rows is staged in LDS once for all of them.
+// read the same rows, so a wave takes several heads of a token at once and every cached element it loads serves them all.
 // The softmax may hold a sink: a per-head number whose exponential joins the denominator without a value.
 // Scores, weights and sums are 32-bit whatever the cache holds.
 #include "common.h"
@@ -22,15 +22,17 @@ __device__ __forceinline__ void store_from_float(void* base, size_t index, int c
 // out[row, head, n] = sum_k x[row, head, k] * w[head, n, k] (* sigmoid(gate[row, head * N + n]), the gate's rows gate_row_stride apart):
 // one small product per head.
 // A block takes HEADS_ROWS rows of one head: their x in LDS (32-bit), a thread an output column at a time, its W row read in
-// 16-byte pieces where K allows.
+// 16-byte pieces where K allows; with fewer columns than threads the threads cut K among themselves and add up through LDS.
 constexpr int HEADS_ROWS = 16;
 
 template <typename WT>
 __global__ __launch_bounds__(256) void heads_linear_kernel(const void* __restrict__ x, int x_code, int x_row_stride, int x_head_stride,
                                                            const WT* __restrict__ w, const void* __restrict__ gate, int gate_code, int gate_row_stride,
                                                            void* __restrict__ out, int out_code, int out_row_stride, int out_head_stride,
-                                                           int n_rows, int N, int K) {
-    extern __shared__ float x_tile[];   // [HEADS_ROWS][K]
+                                                           int n_rows, int N, int K, int cols) {
+    extern __shared__ float heads_lds[];   // x_tile [HEADS_ROWS][K], then the partial sums [slices - 1][cols][HEADS_ROWS]
+    float* x_tile = heads_lds;
+    float* partial = heads_lds + HEADS_ROWS * K;
     const int head = blockIdx.y, row0 = blockIdx.x * HEADS_ROWS;
     const int rows = min(HEADS_ROWS, n_rows - row0);
     for (int i = threadIdx.x; i < HEADS_ROWS * K; i += blockDim.x) {
@@ -40,164 +42,232 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const void* __restric
     __syncthreads();
     constexpr int VEC = 16 / (int)sizeof(WT);
     const bool pieces = K % VEC == 0;
-    for (int n = threadIdx.x; n < N; n += blockDim.x) {
-        const WT* w_row = w + ((size_t)head * N + n) * K;
+    // `cols` threads take a column each; where the block has more threads than that, they cut K into slices
+    const int slices = blockDim.x / cols, column = threadIdx.x % cols, slice = threadIdx.x / cols;
+    const int per_slice = ceil_div(ceil_div(K, slices), VEC) * VEC;
+    const int k_lo = min(K, slice * per_slice), k_hi = min(K, k_lo + per_slice);
+    for (int n0 = 0; n0 < N; n0 += cols) {
+        const int n = n0 + column;
         float acc[HEADS_ROWS];
 #pragma unroll
         for (int r = 0; r < HEADS_ROWS; r++) acc[r] = 0.0f;
-        if (pieces) {
-            for (int k = 0; k < K; k += VEC) {
-                Vec16 piece = *reinterpret_cast<const Vec16*>(w_row + k);
-                const WT* e = reinterpret_cast<const WT*>(&piece);
+        if (n < N) {
+            const WT* w_row = w + ((size_t)head * N + n) * K;
+            if (pieces) {
+                for (int k = k_lo; k < k_hi; k += VEC) {
+                    Vec16 piece = *reinterpret_cast<const Vec16*>(w_row + k);
+                    const WT* e = reinterpret_cast<const WT*>(&piece);
 #pragma unroll
-                for (int j = 0; j < VEC; j++) {
-                    const float wv = to_float(e[j]);
+                    for (int j = 0; j < VEC; j++) {
+                        const float wv = to_float(e[j]);
 #pragma unroll
-                    for (int r = 0; r < HEADS_ROWS; r++) acc[r] += wv * x_tile[r * K + k + j];
+                        for (int r = 0; r < HEADS_ROWS; r++) acc[r] += wv * x_tile[r * K + k + j];
+                    }
+                }
+            } else {
+                for (int k = k_lo; k < k_hi; k++) {
+                    const float wv = to_float(w_row[k]);
+#pragma unroll
+                    for (int r = 0; r < HEADS_ROWS; r++) acc[r] += wv * x_tile[r * K + k];
                 }
             }
-        } else {
-            for (int k = 0; k < K; k++) {
-                const float wv = to_float(w_row[k]);
-#pragma unroll
-                for (int r = 0; r < HEADS_ROWS; r++) acc[r] += wv * x_tile[r * K + k];
-            }
         }
-        for (int r = 0; r < rows; r++) {
-            float value = acc[r];
-            if (gate) {
-                const float g = load_as_float(gate, (size_t)(row0 + r) * gate_row_stride + (size_t)head * N + n, gate_code);
-                value *= 1.0f / (1.0f + expf(-g));
+        if (slices > 1) {   // uniform over the block
+            if (slice > 0)
+#pragma unroll
+                for (int r = 0; r < HEADS_ROWS; r++) partial[((slice - 1) * cols + column) * HEADS_ROWS + r] = acc[r];
+            __syncthreads();
+            if (slice == 0)
+                for (int other = 1; other < slices; other++)
+#pragma unroll
+                    for (int r = 0; r < HEADS_ROWS; r++) acc[r] += partial[((other - 1) * cols + column) * HEADS_ROWS + r];
+            __syncthreads();
+        }
+        if (slice == 0 && n < N) {
+            for (int r = 0; r < rows; r++) {
+                float value = acc[r];
+                if (gate) {
+                    const float g = load_as_float(gate, (size_t)(row0 + r) * gate_row_stride + (size_t)head * N + n, gate_code);
+                    value *= 1.0f / (1.0f + expf(-g));
+                }
+                store_from_float(out, (size_t)(row0 + r) * out_row_stride + (size_t)head * out_head_stride + n, out_code, value);
             }
-            store_from_float(out, (size_t)(row0 + r) * out_row_stride + (size_t)head * out_head_stride + n, out_code, value);
         }
     }
 }
 
-constexpr int LATENT_WAVES = 16;      // heads a block takes
-constexpr int LATENT_TILE = 32;       // cached rows a tile holds
-constexpr int LATENT_VALUE_REGS = 8;  // a lane's share of the latent: ranks up to 512
+constexpr int LATENT_ROWS = 4;   // rows of the batch a block takes, a wave each
 
-// A block per (row of the batch, run of its keys, 16 heads). q [rows, n_heads, D] (32-bit: the folded query, the rotated
-// part, zeros), pages [num_pages, page_size, D], D a multiple of 16 bytes. The first R elements of a cached row are the
-// latent (also the value). gridDim.y = 1: out [rows, n_heads, R] (32-bit) holds the finished sums, sink included. More runs:
-// every run leaves its unnormalised sums, maximum and weight in parts [rows, n_heads, runs, R + 2], which latent_merge_kernel puts together.
 template <typename T>
-__global__ __launch_bounds__(64 * LATENT_WAVES) void latent_attention_kernel(
+__device__ __forceinline__ float piece_element(const Vec16& piece, int e) {
+    if constexpr (sizeof(T) == 2) {
+        const uint32_t word = piece.w[e / 2];
+        return __builtin_bit_cast(float, (e & 1) ? (word & 0xffff0000u) : (word << 16));
+    } else {
+        return __builtin_bit_cast(float, piece.w[e]);
+    }
+}
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// A wave per (row of the batch, run of its keys, HG heads). q [rows, n_heads, D] (32-bit: the folded query, the rotated part,
+// zeros), pages [num_pages, page_size, D], D a multiple of 16 bytes; the first R elements of a cached row are the latent
+// (also the value), R <= 64 * RV.
+//
+// All heads of a row read the same cached rows, so a wave takes HG heads at once: for the scores a lane takes a key and
+// reads its row in 16-byte pieces, each element of which meets the HG queries' elements, which are the same for every lane
+// (they come through the scalar unit); for the weighted sum a lane takes pairs of latent elements, and a key's weight for
+// each head is read out of the lane that holds it. So a cached element costs one load and HG multiply-adds. Keys in
+// tiles of 64 with online softmax statistics per head. n_runs = 1: out [rows, n_heads, R] holds the finished sums, sink
+// included. More runs: every run leaves its unnormalised sums, maximum and weight in parts [rows, n_heads, runs, R + 2].
+template <typename T, int HG, int RV>
+__global__ __launch_bounds__(64 * LATENT_ROWS) void latent_attention_kernel(
     const float* __restrict__ q, const T* __restrict__ pages, const float* __restrict__ sinks, float* __restrict__ out, float* __restrict__ parts,
     const int* __restrict__ token_request, const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks,
-    int n_heads, int R, int D, int page_size, float scale, int run_length) {
-    extern __shared__ float lds[];
-    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-    const int token = blockIdx.x, run = blockIdx.y, n_runs = gridDim.y;
-    const int head = blockIdx.z * LATENT_WAVES + wave;
+    int n_rows, int n_heads, int R, int D, int page_size, float scale, int run_length) {
+    const int lane = threadIdx.x % WAVE;
+    const int token = blockIdx.x * LATENT_ROWS + __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    if (token >= n_rows) return;
+    const int run = blockIdx.y, n_runs = gridDim.y, head0 = blockIdx.z * HG;
     const int request = token_request[token];
-    const bool live_head = head < n_heads;
-    const int row_dwords = D * (int)sizeof(T) / 4 + 1;   // an odd stride: a lane per cached row reads without bank conflicts
-    float* q_lds = lds;                                                  // [LATENT_WAVES][D]
-    uint32_t* tile = reinterpret_cast<uint32_t*>(lds + LATENT_WAVES * D);   // [LATENT_TILE][row_dwords]
-    float* weights = reinterpret_cast<float*>(tile + LATENT_TILE * row_dwords);   // [LATENT_WAVES][LATENT_TILE]
 
-    float o[LATENT_VALUE_REGS];
+    float o[HG][RV], top[HG], weight[HG];
 #pragma unroll
-    for (int r = 0; r < LATENT_VALUE_REGS; r++) o[r] = 0.0f;
-    float running_max = -INFINITY, running_sum = 0.0f;
+    for (int h = 0; h < HG; h++) {
+        top[h] = -INFINITY;
+        weight[h] = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RV; r++) o[h][r] = 0.0f;
+    }
 
-    if (request >= 0) {   // uniform over the block
+    if (request >= 0) {
         const int position = positions[token];
-        const int first_key = run * run_length, last_key = min(position, first_key + run_length - 1);
+        const int first_key = run * run_length;
+        const int last_key = run == n_runs - 1 ? position : min(position, first_key + run_length - 1);   // the last run is open-ended
         const int* table = block_tables + (size_t)request * max_blocks;
-        if (live_head)
-            for (int d = lane; d < D; d += WAVE) q_lds[wave * D + d] = q[((size_t)token * n_heads + head) * D + d] * scale;
+        const float* q_head[HG];   // the same for every lane
+#pragma unroll
+        for (int h = 0; h < HG; h++) q_head[h] = q + ((size_t)token * n_heads + min(head0 + h, n_heads - 1)) * D;
         constexpr int VEC = 16 / (int)sizeof(T);
-        const int pieces_per_row = D / VEC;
-        for (int tile0 = first_key; tile0 <= last_key; tile0 += LATENT_TILE) {
-            __syncthreads();   // the tile before has been read by every wave (and q_lds is written)
-            for (int i = threadIdx.x; i < LATENT_TILE * pieces_per_row; i += blockDim.x) {
-                const int j = i / pieces_per_row, piece = i % pieces_per_row;
-                const int key = min(tile0 + j, last_key);
-                const int page = table[key / page_size];
-                const Vec16 v = *reinterpret_cast<const Vec16*>(pages + ((size_t)page * page_size + key % page_size) * D + piece * VEC);
-                uint32_t* at = tile + j * row_dwords + piece * 4;
-                at[0] = v.w[0]; at[1] = v.w[1]; at[2] = v.w[2]; at[3] = v.w[3];
-            }
-            __syncthreads();
-            if (!live_head) continue;
-            // scores: two lanes a cached row, each half of the elements
-            const int j = lane % LATENT_TILE, part = lane / LATENT_TILE;
-            const T* row = reinterpret_cast<const T*>(tile + j * row_dwords);
-            const int half = (D / 2 + 1) & ~1;   // an even split, so that pairs of bfloat16 stay whole
-            const int d_lo = part * half, d_hi = min(D, d_lo + half);
-            float dot = 0.0f;
-            const float* my_q = q_lds + wave * D;
-            if constexpr (sizeof(T) == 2) {
-                for (int d = d_lo; d < d_hi; d += 2) {
-                    const uint32_t pair = *reinterpret_cast<const uint32_t*>(row + d);
-                    dot += my_q[d] * __builtin_bit_cast(float, pair << 16) + my_q[d + 1] * __builtin_bit_cast(float, pair & 0xffff0000u);
-                }
-            } else {
-                for (int d = d_lo; d < d_hi; d++) dot += my_q[d] * to_float(row[d]);
-            }
-            dot += __shfl_xor(dot, LATENT_TILE, WAVE);
-            const bool valid = tile0 + j <= last_key;
-            const float score = valid ? dot : -INFINITY;
-            const float new_max = fmaxf(running_max, wave_max(score));
-            const float p = valid ? expf(score - new_max) : 0.0f;
-            const float rescale = expf(running_max - new_max);   // the first tile of a run always holds a key: new_max is finite
-            running_sum = running_sum * rescale + wave_sum(part == 0 ? p : 0.0f);
-            running_max = new_max;
-            if (part == 0) weights[wave * LATENT_TILE + j] = p;
-            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            const int in_tile = min(LATENT_TILE, last_key - tile0 + 1);
+        for (int tile0 = first_key; tile0 <= last_key; tile0 += WAVE) {
+            const bool valid = tile0 + lane <= last_key;
+            const int key = min(tile0 + lane, last_key);
+            const int slot = table[key / page_size] * page_size + key % page_size;
+            const T* row = pages + (size_t)slot * D;
+            float s[HG];
 #pragma unroll
-            for (int r = 0; r < LATENT_VALUE_REGS; r++) {
-                const int d = lane + r * WAVE;
-                if (d < R) {
-                    float sum = o[r] * rescale;
-                    for (int k = 0; k < in_tile; k++)
-                        sum += weights[wave * LATENT_TILE + k] * to_float(reinterpret_cast<const T*>(tile + k * row_dwords)[d]);
-                    o[r] = sum;
+            for (int h = 0; h < HG; h++) s[h] = 0.0f;
+            // four pieces of the lane's row are asked for at a time, so that their ways from memory overlap
+            int d0 = 0;
+            for (; d0 + 4 * VEC <= D; d0 += 4 * VEC) {
+                Vec16 pieces[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) pieces[u] = *reinterpret_cast<const Vec16*>(row + d0 + u * VEC);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) {
+                        const float k = piece_element<T>(pieces[u], e);
+#pragma unroll
+                        for (int h = 0; h < HG; h++) s[h] = __builtin_fmaf(q_head[h][d0 + u * VEC + e], k, s[h]);
+                    }
+            }
+            for (; d0 < D; d0 += VEC) {
+                const Vec16 piece = *reinterpret_cast<const Vec16*>(row + d0);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    const float k = piece_element<T>(piece, e);
+#pragma unroll
+                    for (int h = 0; h < HG; h++) s[h] = __builtin_fmaf(q_head[h][d0 + e], k, s[h]);
                 }
             }
-            __builtin_amdgcn_wave_barrier();
-        }
-    }
-    if (!live_head) return;
-    if (n_runs == 1) {
-        float inverse = 0.0f;
-        if (request >= 0) {
-            float total = running_sum;
-            if (sinks) {   // the sink joins the denominator once: measured from the larger of the two
-                const float sink = sinks[head], top = fmaxf(running_max, sink);
-                const float shrink = expf(running_max - top);
-                total = running_sum * shrink + expf(sink - top);
-                inverse = shrink / total;
-            } else {
-                inverse = 1.0f / total;
+            float p[HG];
+#pragma unroll
+            for (int h = 0; h < HG; h++) {
+                const float score = valid ? s[h] * scale : -INFINITY;
+                const float new_top = fmaxf(top[h], wave_max_total(score));   // finite: a tile holds at least one key
+                p[h] = valid ? expf(score - new_top) : 0.0f;
+                const float rescale = expf(top[h] - new_top);
+                weight[h] = weight[h] * rescale + wave_total(p[h]);
+                top[h] = new_top;
+#pragma unroll
+                for (int r = 0; r < RV; r++) o[h][r] *= rescale;
+            }
+            // the weighted sum: a lane takes elements 2 * lane + 128 * r2 and the one behind it. Eight keys' values are asked
+            // for at a time; lanes beyond the tile's keys hold a weight of zero and the place of a key that exists
+            const int in_tile = min(WAVE, last_key - tile0 + 1);
+            constexpr int KEYS = 8;
+            for (int j0 = 0; j0 < in_tile; j0 += KEYS) {
+                float v[KEYS][RV];
+#pragma unroll
+                for (int u = 0; u < KEYS; u++) {
+                    const T* value_row = pages + (size_t)__builtin_amdgcn_readlane(slot, j0 + u) * D;
+#pragma unroll
+                    for (int r2 = 0; r2 < RV / 2; r2++) {
+                        const int d = min(2 * lane + 2 * WAVE * r2, D - 2);   // beyond R: read, and never stored
+                        if constexpr (sizeof(T) == 2) {
+                            const uint32_t pair = *reinterpret_cast<const uint32_t*>(value_row + d);
+                            v[u][2 * r2] = __builtin_bit_cast(float, pair << 16);
+                            v[u][2 * r2 + 1] = __builtin_bit_cast(float, pair & 0xffff0000u);
+                        } else {
+                            const float2 pair = *reinterpret_cast<const float2*>(value_row + d);
+                            v[u][2 * r2] = pair.x;
+                            v[u][2 * r2 + 1] = pair.y;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < KEYS; u++)
+#pragma unroll
+                    for (int h = 0; h < HG; h++) {
+                        const float pj = lane_value(p[h], j0 + u);
+#pragma unroll
+                        for (int r = 0; r < RV; r++) o[h][r] = __builtin_fmaf(pj, v[u][r], o[h][r]);
+                    }
             }
         }
-        float* out_row = out + ((size_t)token * n_heads + head) * R;
+    }
 #pragma unroll
-        for (int r = 0; r < LATENT_VALUE_REGS; r++) {
-            const int d = lane + r * WAVE;
-            if (d < R) out_row[d] = o[r] * inverse;
+    for (int h = 0; h < HG; h++) {
+        const int head = head0 + h;
+        if (head >= n_heads) break;
+        if (n_runs == 1) {
+            float inverse = 0.0f;
+            if (request >= 0) {
+                if (sinks) {   // the sink joins the denominator once: measured from the larger of the two
+                    const float sink = sinks[head], highest = fmaxf(top[h], sink);
+                    const float shrink = expf(top[h] - highest);
+                    inverse = shrink / (weight[h] * shrink + expf(sink - highest));
+                } else {
+                    inverse = 1.0f / weight[h];
+                }
+            }
+            float* out_row = out + ((size_t)token * n_heads + head) * R;
+#pragma unroll
+            for (int r = 0; r < RV; r++) {
+                const int d = 2 * lane + 2 * WAVE * (r / 2) + (r & 1);
+                if (d < R) out_row[d] = o[h][r] * inverse;
+            }
+        } else {
+            float* mine = parts + (((size_t)token * n_heads + head) * n_runs + run) * (R + 2);
+#pragma unroll
+            for (int r = 0; r < RV; r++) {
+                const int d = 2 * lane + 2 * WAVE * (r / 2) + (r & 1);
+                if (d < R) mine[d] = o[h][r];
+            }
+            if (lane == 0) {
+                mine[R] = top[h];   // -inf and 0 for a run without keys
+                mine[R + 1] = weight[h];
+            }
         }
-        return;
-    }
-    float* mine = parts + (((size_t)token * n_heads + head) * n_runs + run) * (R + 2);
-#pragma unroll
-    for (int r = 0; r < LATENT_VALUE_REGS; r++) {
-        const int d = lane + r * WAVE;
-        if (d < R) mine[d] = o[r];
-    }
-    if (lane == 0) {
-        mine[R] = running_max;   // -inf and 0 for a run without keys
-        mine[R + 1] = running_sum;
     }
 }
 
 // out[row, head] = sum_p o_p e^(m_p - M) / (sum_p l_p e^(m_p - M) + e^(sink - M)) over the runs of a (row, head); a wave each.
+// Lane p takes run p's maximum and weight (and the next 64 runs' after them), so the statistics cost one trip to memory; the
+// sums over the runs are taken four loads at a time.
 __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ parts, const float* __restrict__ sinks,
                                                            const int* __restrict__ token_request, float* __restrict__ out, int n_rows,
                                                            int n_heads, int n_runs, int R) {
@@ -211,27 +281,33 @@ __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restri
         return;
     }
     const float* runs = parts + (size_t)item * n_runs * (R + 2);
-    float top = sinks ? sinks[head] : -INFINITY;
-    for (int p = 0; p < n_runs; p++) top = fmaxf(top, runs[p * (R + 2) + R]);
-    float total = sinks ? expf(sinks[head] - top) : 0.0f;
-    for (int p = 0; p < n_runs; p++) {
-        const float m = runs[p * (R + 2) + R];
-        total += m == -INFINITY ? 0.0f : runs[p * (R + 2) + R + 1] * expf(m - top);
+    const float sink = sinks ? sinks[head] : -INFINITY;
+    float my_top = -INFINITY;
+    for (int p = lane; p < n_runs; p += WAVE) my_top = fmaxf(my_top, runs[(size_t)p * (R + 2) + R]);
+    const float top = fmaxf(sink, wave_max_total(my_top));   // finite: the first run always holds a key
+    float my_total = 0.0f;
+    for (int p = lane; p < n_runs; p += WAVE) {
+        const float m = runs[(size_t)p * (R + 2) + R];
+        my_total += m == -INFINITY ? 0.0f : runs[(size_t)p * (R + 2) + R + 1] * expf(m - top);
     }
+    const float total = wave_total(my_total) + (sinks ? expf(sink - top) : 0.0f);
     const float inverse = 1.0f / total;
-    for (int d = lane; d < R; d += WAVE) {
+    for (int d0 = 0; d0 < R; d0 += WAVE) {
+        const int d = min(d0 + lane, R - 1);
         float sum = 0.0f;
-        for (int p = 0; p < n_runs; p++) {
-            const float m = runs[p * (R + 2) + R];
-            sum += m == -INFINITY ? 0.0f : runs[p * (R + 2) + d] * expf(m - top);
+        for (int p0 = 0; p0 < n_runs; p0 += 4) {
+            float o[4], m[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const size_t at = (size_t)min(p0 + u, n_runs - 1) * (R + 2);
+                o[u] = runs[at + d];
+                m[u] = runs[at + R];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) sum += p0 + u < n_runs && m[u] != -INFINITY ? o[u] * expf(m[u] - top) : 0.0f;
         }
-        out_row[d] = sum * inverse;
+        if (d0 + lane < R) out_row[d] = sum * inverse;
     }
-}
-
-size_t latent_lds_bytes(int D, int element) {
-    const int row_dwords = D * element / 4 + 1;
-    return (size_t)LATENT_WAVES * D * 4 + (size_t)LATENT_TILE * row_dwords * 4 + (size_t)LATENT_WAVES * LATENT_TILE * 4;
 }
 
 template <typename KernelT>
@@ -245,6 +321,43 @@ int allow_lds(KernelT kernel, size_t bytes, const char* what) {
     return 0;
 }
 
+// Heads a wave takes at once: all of them in equal groups where the count allows, else groups of which the last is not full.
+int latent_head_group(int n_heads) {
+    if (n_heads % 8 == 0) return 8;
+    if (n_heads % 6 == 0) return 6;
+    if (n_heads % 4 == 0) return 4;
+    return n_heads <= 4 ? 4 : (n_heads <= 6 ? 6 : 8);
+}
+
+struct LatentArgs {
+    const float* q; const void* pages; const float* sinks; float* out; float* parts; const int* token_request; const int* positions;
+    const int* block_tables; int max_blocks, n_rows, n_heads, R, D, page_size; float scale; int n_runs, run_length; hipStream_t stream;
+};
+
+template <typename T, int HG, int RV>
+void launch_latent(const LatentArgs& a) {
+    dim3 grid(ceil_div(a.n_rows, LATENT_ROWS), a.n_runs, ceil_div(a.n_heads, HG));
+    latent_attention_kernel<T, HG, RV><<<grid, 64 * LATENT_ROWS, 0, a.stream>>>(a.q, (const T*)a.pages, a.sinks, a.out, a.parts, a.token_request, a.positions,
+                                                                                a.block_tables, a.max_blocks, a.n_rows, a.n_heads, a.R, a.D, a.page_size,
+                                                                                a.scale, a.run_length);
+}
+
+template <typename T, int HG>
+void launch_latent_rv(const LatentArgs& a) {
+    if (a.R <= 2 * WAVE) launch_latent<T, HG, 2>(a);
+    else if (a.R <= 4 * WAVE) launch_latent<T, HG, 4>(a);
+    else launch_latent<T, HG, 8>(a);
+}
+
+template <typename T>
+void launch_latent_hg(const LatentArgs& a) {
+    switch (latent_head_group(a.n_heads)) {
+        case 4: launch_latent_rv<T, 4>(a); break;
+        case 6: launch_latent_rv<T, 6>(a); break;
+        default: launch_latent_rv<T, 8>(a); break;
+    }
+}
+
 }  // namespace
 
 MLLM_API int mllm_heads_linear(const void* x, int x_dtype, int x_row_stride, int x_head_stride, const void* w, int w_dtype, const void* gate,
@@ -256,20 +369,20 @@ MLLM_API int mllm_heads_linear(const void* x, int x_dtype, int x_row_stride, int
                  "heads_linear: rows are too short for the heads");
     for (int code : {x_dtype, w_dtype, out_dtype}) MLLM_REQUIRE(code == MLLM_F32 || code == MLLM_BF16, "heads_linear: unknown dtype %d", code);
     MLLM_REQUIRE(gate == nullptr || ((gate_dtype == MLLM_F32 || gate_dtype == MLLM_BF16) && gate_row_stride >= n_heads * N), "heads_linear: a gate of unknown element type or with rows too short");
-    const size_t lds = (size_t)HEADS_ROWS * K * sizeof(float);
+    const int threads = 256, cols = N > 128 ? 256 : (N > 64 ? 128 : 64);
+    const size_t lds = ((size_t)HEADS_ROWS * K + (size_t)(threads / cols - 1) * cols * HEADS_ROWS) * sizeof(float);
     MLLM_REQUIRE(lds <= 64 * 1024, "heads_linear: K = %d is more than a block holds in LDS", K);
     if (n_rows == 0) return 0;
     dim3 grid(ceil_div(n_rows, HEADS_ROWS), n_heads);
-    const int threads = N >= 256 ? 256 : (N > 64 ? 128 : 64);
     mllm_count_kernel(MLLM_K_HEADS_LINEAR);
     if (w_dtype == MLLM_F32) {
         if (allow_lds(heads_linear_kernel<float>, lds, "heads_linear")) return 1;
         heads_linear_kernel<float><<<grid, threads, lds, stream>>>(x, x_dtype, x_row_stride, x_head_stride, (const float*)w, gate, gate_dtype, gate_row_stride, out, out_dtype,
-                                                                   out_row_stride, out_head_stride, n_rows, N, K);
+                                                                   out_row_stride, out_head_stride, n_rows, N, K, cols);
     } else {
         if (allow_lds(heads_linear_kernel<bf16_t>, lds, "heads_linear")) return 1;
         heads_linear_kernel<bf16_t><<<grid, threads, lds, stream>>>(x, x_dtype, x_row_stride, x_head_stride, (const bf16_t*)w, gate, gate_dtype, gate_row_stride, out, out_dtype,
-                                                                    out_row_stride, out_head_stride, n_rows, N, K);
+                                                                    out_row_stride, out_head_stride, n_rows, N, K, cols);
     }
     return mllm_check_launch("heads_linear");
 }
@@ -277,8 +390,11 @@ MLLM_API int mllm_heads_linear(const void* x, int x_dtype, int x_row_stride, int
 // Whether the latent attention kernel takes rows of D elements of which R are the latent.
 MLLM_API int mllm_latent_attention_supported(int R, int D, int dtype) {
     const int element = dtype == MLLM_F32 ? 4 : 2;
-    return R > 0 && R <= D && R <= WAVE * LATENT_VALUE_REGS && (D * element) % 16 == 0 && latent_lds_bytes(D, element) <= 160 * 1024 - 1024;
+    return R > 0 && R <= D && R <= 8 * WAVE && (D * element) % 16 == 0;
 }
+
+// How many heads a wave of the latent attention kernel takes at once (its launches have rows / 4 x runs x heads / this many blocks).
+MLLM_API int mllm_latent_attention_head_group(int n_heads) { return n_heads > 0 ? latent_head_group(n_heads) : 0; }
 
 MLLM_API int mllm_latent_attention(const float* q, const void* pages, const float* sinks, float* out, float* parts, const int* token_request,
                                    const int* positions, const int* block_tables, int max_blocks, int n_rows, int n_heads, int R, int D,
@@ -288,22 +404,12 @@ MLLM_API int mllm_latent_attention(const float* q, const void* pages, const floa
     MLLM_REQUIRE(mllm_latent_attention_supported(R, D, dtype), "latent_attention: no kernel for rows of %d elements with a latent of %d", D, R);
     MLLM_REQUIRE(n_runs >= 1 && n_runs <= 65535 && run_length >= 1, "latent_attention: bad runs");
     MLLM_REQUIRE(n_runs == 1 || parts != nullptr, "latent_attention: runs need room for their sums");
-    MLLM_REQUIRE(n_runs == 1 || (long long)n_runs * run_length >= (long long)max_blocks * page_size, "latent_attention: the runs do not cover the longest sequence");
     if (n_rows == 0) return 0;
-    const size_t lds = latent_lds_bytes(D, dtype == MLLM_F32 ? 4 : 2);
-    dim3 grid(n_rows, n_runs, ceil_div(n_heads, LATENT_WAVES));
-    const int threads = 64 * (n_heads < LATENT_WAVES ? n_heads : LATENT_WAVES);
     if (n_runs == 1) run_length = 1 << 30;
+    const LatentArgs args{q, pages, sinks, out, parts, token_request, positions, block_tables, max_blocks, n_rows, n_heads, R, D, page_size, scale, n_runs, run_length, stream};
     mllm_count_kernel(MLLM_K_LATENT_ATTENTION);
-    if (dtype == MLLM_F32) {
-        if (allow_lds(latent_attention_kernel<float>, lds, "latent_attention")) return 1;
-        latent_attention_kernel<float><<<grid, threads, lds, stream>>>(q, (const float*)pages, sinks, out, parts, token_request, positions, block_tables,
-                                                                       max_blocks, n_heads, R, D, page_size, scale, run_length);
-    } else {
-        if (allow_lds(latent_attention_kernel<bf16_t>, lds, "latent_attention")) return 1;
-        latent_attention_kernel<bf16_t><<<grid, threads, lds, stream>>>(q, (const bf16_t*)pages, sinks, out, parts, token_request, positions, block_tables,
-                                                                        max_blocks, n_heads, R, D, page_size, scale, run_length);
-    }
+    if (dtype == MLLM_F32) launch_latent_hg<float>(args);
+    else launch_latent_hg<bf16_t>(args);
     int status = mllm_check_launch("latent_attention");
     if (status || n_runs == 1) return status;
     const long long items = (long long)n_rows * n_heads;

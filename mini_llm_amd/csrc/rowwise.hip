@@ -28,40 +28,53 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
     if (row >= n_rows) return;
     const int source = row_index ? row_index[row] : row;
     const size_t in_at = (size_t)source * width, out_at = (size_t)row * width;
-    float kept[REGS > 0 ? REGS : 1];
-    float squares = 0.0f;
+    const float plus = one_plus ? 1.0f : 0.0f;
     if constexpr (REGS > 0) {
+        // everything is asked for at once, from clamped places, so that the wave waits for memory once
+        float kept[REGS], added[REGS], gains[REGS];
 #pragma unroll
         for (int r = 0; r < REGS; r++) {
-            const int i = lane + r * WAVE;
-            float h = 0.0f;
-            if (i < width) {
-                h = alpha * x[in_at + i];
-                if (y) h += load_as_float(y, in_at + i, y_code);
+            const int i = min(lane + r * WAVE, width - 1);
+            kept[r] = x[in_at + i];
+            gains[r] = weight[i];
+        }
+        if (y) {
+            if (y_code == MLLM_F32) {
+#pragma unroll
+                for (int r = 0; r < REGS; r++) added[r] = reinterpret_cast<const float*>(y)[in_at + min(lane + r * WAVE, width - 1)];
+            } else {
+#pragma unroll
+                for (int r = 0; r < REGS; r++) added[r] = to_float(reinterpret_cast<const bf16_t*>(y)[in_at + min(lane + r * WAVE, width - 1)]);
             }
+        } else {
+#pragma unroll
+            for (int r = 0; r < REGS; r++) added[r] = 0.0f;
+        }
+        float squares = 0.0f;
+#pragma unroll
+        for (int r = 0; r < REGS; r++) {
+            const float h = lane + r * WAVE < width ? alpha * kept[r] + added[r] : 0.0f;
             kept[r] = h;
             squares += h * h;
         }
-    } else {
-        for (int i = lane; i < width; i += WAVE) {
-            float h = alpha * x[in_at + i];
-            if (y) h += load_as_float(y, in_at + i, y_code);
-            squares += h * h;
-        }
-    }
-    const float inverse = 1.0f / sqrtf(wave_sum(squares) / (float)width + eps);
-    const float plus = one_plus ? 1.0f : 0.0f;
-    if constexpr (REGS > 0) {
+        const float inverse = 1.0f / sqrtf(wave_total(squares) / (float)width + eps);
 #pragma unroll
         for (int r = 0; r < REGS; r++) {
             const int i = lane + r * WAVE;
             if (i < width) {
-                const float value = kept[r] * inverse * (plus + weight[i]);
+                const float value = kept[r] * inverse * (plus + gains[r]);
                 if (stream) stream[out_at + i] = value;
                 if (rows) store_from_float(rows, out_at + i, rows_code, value);
             }
         }
     } else {
+        float squares = 0.0f;
+        for (int i = lane; i < width; i += WAVE) {
+            float h = alpha * x[in_at + i];
+            if (y) h += load_as_float(y, in_at + i, y_code);
+            squares += h * h;
+        }
+        const float inverse = 1.0f / sqrtf(wave_total(squares) / (float)width + eps);
         for (int i = lane; i < width; i += WAVE) {
             float h = alpha * x[in_at + i];
             if (y) h += load_as_float(y, in_at + i, y_code);
@@ -190,15 +203,33 @@ __global__ __launch_bounds__(256) void latent_rows_kernel(const T* __restrict__ 
     for (int i = 2 * half + lane; i < row_size - rank; i += WAVE) out[rank + i] = i < rot ? in[rank + i] : from_float<T>(0.0f);
 }
 
-// out[row, j] = silu(both[row, j]) * both[row, inner + j]: the two halves of a fused gate / up product.
-template <typename T>
-__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ both, T* __restrict__ out, long long n, int inner) {
-    const long long at = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (at >= n) return;
-    const long long row = at / inner;
-    const int j = (int)(at % inner);
-    const float a = to_float(both[row * 2 * inner + j]), b = to_float(both[row * 2 * inner + inner + j]);
-    out[at] = from_float<T>(a / (1.0f + expf(-a)) * b);
+// out[row, j] = silu(both[row, j]) * both[row, inner + j]: the two halves of a fused gate / up product. A thread takes a
+// 16-byte piece of each half where the rows are whole pieces (PIECES), else an element.
+template <typename T, bool PIECES>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ both, T* __restrict__ out, int inner) {
+    constexpr int VEC = PIECES ? 16 / (int)sizeof(T) : 1;
+    const int j = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (j >= inner) return;
+    const size_t row = blockIdx.y;
+    const T* a_at = both + row * 2 * inner + j;
+    const T* b_at = a_at + inner;
+    T* out_at = out + row * inner + j;
+    if constexpr (PIECES) {
+        const Vec16 a = *reinterpret_cast<const Vec16*>(a_at), b = *reinterpret_cast<const Vec16*>(b_at);
+        Vec16 result;
+        const T* ae = reinterpret_cast<const T*>(&a);
+        const T* be = reinterpret_cast<const T*>(&b);
+        T* re = reinterpret_cast<T*>(&result);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const float av = to_float(ae[e]);
+            re[e] = from_float<T>(av / (1.0f + expf(-av)) * to_float(be[e]));
+        }
+        *reinterpret_cast<Vec16*>(out_at) = result;
+    } else {
+        const float av = to_float(*a_at);
+        *out_at = from_float<T>(av / (1.0f + expf(-av)) * to_float(*b_at));
+    }
 }
 
 }  // namespace
@@ -215,6 +246,7 @@ MLLM_API int mllm_rms_norm(const float* x, const void* y, int y_dtype, float alp
     mllm_count_kernel(MLLM_K_RMS_NORM);
 #define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width)
     if (width <= 256) LAUNCH(4);
+    else if (width <= 512) LAUNCH(8);
     else if (width <= 1024) LAUNCH(16);
     else if (width <= 2048) LAUNCH(32);
     else LAUNCH(0);
@@ -274,14 +306,30 @@ MLLM_API int mllm_latent_rows(const void* q, int q_stride, const void* dkv, int 
     return mllm_check_launch("latent_rows");
 }
 
+template <typename T>
+void launch_silu_mul(const void* both, void* out, int n_rows, int inner, hipStream_t stream) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (inner % VEC == 0) {
+        dim3 grid(ceil_div(inner / VEC, 256), n_rows);
+        silu_mul_kernel<T, true><<<grid, 256, 0, stream>>>((const T*)both, (T*)out, inner);
+    } else {
+        dim3 grid(ceil_div(inner, 256), n_rows);
+        silu_mul_kernel<T, false><<<grid, 256, 0, stream>>>((const T*)both, (T*)out, inner);
+    }
+}
+
 MLLM_API int mllm_silu_mul(const void* both, void* out, int n_rows, int inner, int dtype, hipStream_t stream) {
-    MLLM_REQUIRE(n_rows >= 0 && inner > 0, "silu_mul: bad sizes");
+    MLLM_REQUIRE(n_rows >= 0 && n_rows <= 65535 * 64 && inner > 0, "silu_mul: bad sizes");
+    MLLM_REQUIRE(dtype == MLLM_F32 || dtype == MLLM_BF16, "silu_mul: unknown dtype %d", dtype);
     if (n_rows == 0) return 0;
-    const long long n = (long long)n_rows * inner;
-    const int blocks = (int)((n + 255) / 256);
     mllm_count_kernel(MLLM_K_SILU_MUL);
-    if (dtype == MLLM_F32) silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)both, (float*)out, n, inner);
-    else if (dtype == MLLM_BF16) silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)both, (bf16_t*)out, n, inner);
-    else MLLM_REQUIRE(false, "silu_mul: unknown dtype %d", dtype);
+    for (int row0 = 0; row0 < n_rows; row0 += 65535) {   // the grid's second dimension holds 65,535 rows
+        const int rows = n_rows - row0 < 65535 ? n_rows - row0 : 65535;
+        const size_t element = dtype == MLLM_F32 ? 4 : 2;
+        const char* in_at = (const char*)both + (size_t)row0 * 2 * inner * element;
+        char* out_at = (char*)out + (size_t)row0 * inner * element;
+        if (dtype == MLLM_F32) launch_silu_mul<float>(in_at, out_at, rows, inner, stream);
+        else launch_silu_mul<bf16_t>(in_at, out_at, rows, inner, stream);
+    }
     return mllm_check_launch("silu_mul");
 }

@@ -923,7 +923,8 @@ def heads_linear(x, weight, out, *, n_heads, k, x_head_stride, n_out=None, gate=
     return out
 
 
-LATENT_RUN_MIN = 256   # cached rows a run of a token's keys should at least hold
+LATENT_RUN_MIN = 64        # cached rows a run of a token's keys should at least hold: a tile of the kernel
+LATENT_TARGET_WAVES = 2048   # waves a launch should have before a token's keys are left whole (eight to a compute unit)
 
 
 def latent_attention_supported(rank: int, row_size: int, dtype) -> bool:
@@ -952,11 +953,10 @@ def latent_attention(q_full, pages, sinks, token_request, positions, block_table
         return out
     reach = block_tables.shape[1] * page_size
     longest = reach if max_len is None else max(1, min(int(max_len), reach))
-    n_runs, units = 1, _compute_units(q_full.device)
-    groups = n * -(-n_heads // 16)
-    while 2 * groups * n_runs <= 2 * units and 2 * n_runs * LATENT_RUN_MIN <= longest:
-        n_runs *= 2
-    run_length = -(-reach // n_runs) if n_runs > 1 else reach
+    # a wave takes a row's keys for a group of heads: few rows with many keys are cut into runs, a wave each
+    waves = n * -(-n_heads // int(library().mllm_latent_attention_head_group(n_heads)))
+    n_runs = max(1, min(LATENT_TARGET_WAVES // waves, longest // LATENT_RUN_MIN, 256))
+    run_length = -(-(-(-longest // n_runs)) // 64) * 64 if n_runs > 1 else reach   # whole tiles; the last run takes whatever lies beyond
     parts = torch.empty((n, n_heads, n_runs, rank + 2), dtype=torch.float32, device=q_full.device) if n_runs > 1 else None
     check(library().mllm_latent_attention(_ptr(q_full), _ptr(pages), _ptr(sinks), _ptr(out), _ptr(parts), _ptr(token_request), _ptr(positions),
                                           _ptr(block_tables), block_tables.shape[1], n, n_heads, int(rank), row_size, page_size, float(scale),

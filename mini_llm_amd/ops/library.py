@@ -53,6 +53,7 @@ _SIGNATURES = {
     "mllm_silu_mul": [P, P, c_int, c_int, c_int, P],
     "mllm_heads_linear": [P, c_int, c_int, c_int, P, c_int, P, c_int, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_latent_attention_supported": [c_int, c_int, c_int],
+    "mllm_latent_attention_head_group": [c_int],
     "mllm_latent_attention": [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
 }
 
