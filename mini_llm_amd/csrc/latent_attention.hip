@@ -310,6 +310,174 @@ __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restri
     }
 }
 
+// The same attention on the matrix cores, for bfloat16 caches whose rows are DK x 16 elements with a latent of up to 32 x RT.
+// A wave takes 32 (token, head) pairs of one request's portion, neighbours in (token, head) order: they all read the same cached
+// rows, so a tile of 32 keys serves 32 pairs in one product. S^T = C Q'^T (a lane's 16-byte piece of its key's row is the
+// operand as it lies in memory; the folded queries, rounded to bfloat16 with the scale folded in, stay in registers for the
+// whole kernel), the statistics per pair in the lane that owns the pair's column, then O^T += C_latent^T P^T with the weights
+// rounded to bfloat16 and the latent elements gathered two at a time (a lane's 32-bit load gives an element to each of two
+// output tiles). Sums, scores and statistics are 32-bit. Runs of keys and the sink as in the kernel above.
+template <int DK, int RT>
+__global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
+    const float* __restrict__ q, const bf16_t* __restrict__ pages, const float* __restrict__ sinks, float* __restrict__ out, float* __restrict__ parts,
+    const int* __restrict__ q_starts, const int* __restrict__ context_lens, const int* __restrict__ block_tables, int max_blocks,
+    int n_heads, int R, int page_size, float scale, int run_length) {
+    constexpr int D = 16 * DK;
+    const int lane = threadIdx.x, lane32 = lane % 32, half = lane / 32;
+    const int request = blockIdx.y, run = blockIdx.z, n_runs = gridDim.z;
+    const int context = context_lens[request];
+    if (context < 0) return;   // a padding request
+    const int q_first = q_starts[request], q_len = q_starts[request + 1] - q_first;
+    const int pair0 = blockIdx.x * 32, n_pairs = q_len * n_heads;
+    if (pair0 >= n_pairs) return;
+    const int pair = pair0 + lane32;
+    const bool pair_valid = pair < n_pairs;
+    const int token = min(pair / n_heads, q_len - 1), head = pair_valid ? pair % n_heads : 0;
+    const int row = q_first + token, position = context + token;
+    const int wave_last_position = context + min(q_len - 1, (pair0 + 31) / n_heads);
+    const int* table = block_tables + (size_t)request * max_blocks;
+
+    bf16x8 q_op[DK];
+    {
+        const float* q_row = q + ((size_t)row * n_heads + head) * D + 8 * half;
+        const float factor = pair_valid ? scale : 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < DK; ks++) {
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(q_row + 16 * ks), hi = *reinterpret_cast<const f32x4*>(q_row + 16 * ks + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                q_op[ks][e] = static_cast<bf16_t>(lo[e] * factor);
+                q_op[ks][4 + e] = static_cast<bf16_t>(hi[e] * factor);
+            }
+        }
+    }
+    f32x16 o[RT];
+#pragma unroll
+    for (int i = 0; i < RT; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[i][v] = 0.0f;
+    float top = -INFINITY, weight = 0.0f;
+
+    const int first_key = run * run_length;
+    const int last_key = run == n_runs - 1 ? wave_last_position : min(wave_last_position, first_key + run_length - 1);
+    for (int kt = first_key; kt <= last_key; kt += 32) {
+        const int key = min(kt + lane32, last_key);
+        const int slot = table[key / page_size] * page_size + key % page_size;
+        const bf16_t* k_row = pages + (size_t)slot * D + 8 * half;
+        bf16x8 k_op[DK];
+#pragma unroll
+        for (int ks = 0; ks < DK; ks++) k_op[ks] = *reinterpret_cast<const bf16x8*>(k_row + 16 * ks);
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; v++) s[v] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < DK; ks++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_op[ks], q_op[ks], s, 0, 0, 0);
+        float tile_top = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int at = kt + 8 * (v / 4) + 4 * half + (v % 4);
+            s[v] = pair_valid && at <= position && at <= last_key ? s[v] : -INFINITY;
+            tile_top = fmaxf(tile_top, s[v]);
+        }
+        tile_top = fmaxf(tile_top, __shfl_xor(tile_top, 32, WAVE));
+        const float new_top = fmaxf(top, tile_top);
+        const float safe_top = new_top == -INFINITY ? 0.0f : new_top;   // a pair none of whose keys has come yet
+        const float rescale = expf(top - safe_top);
+        top = new_top;
+        weight *= rescale;
+#pragma unroll
+        for (int i = 0; i < RT; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) o[i][v] *= rescale;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            s[v] = expf(s[v] - safe_top);
+            weight += s[v];
+        }
+#pragma unroll
+        for (int slab = 0; slab < 2; slab++) {   // 16 keys each: the lane's score registers 8 * slab .. + 7
+            bf16x8 p;
+#pragma unroll
+            for (int e = 0; e < 8; e++) p[e] = static_cast<bf16_t>(s[8 * slab + e]);
+            // the keys those registers belong to: 16 * slab + 4 * half + 0..3 and eight further on; their cached rows
+            const bf16_t* rows_at[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) rows_at[e] = pages + (size_t)__shfl(slot, 16 * slab + 4 * half + (e % 4) + 8 * (e / 4), WAVE) * D;
+#pragma unroll
+            for (int t = 0; t < RT / 2; t++) {
+                const int d = min(64 * t + 2 * lane32, D - 2);
+                uint32_t word[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) word[e] = *reinterpret_cast<const uint32_t*>(rows_at[e] + d);
+                Vec16 even, odd;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    even.w[j] = (word[2 * j] & 0xffffu) | (word[2 * j + 1] << 16);
+                    odd.w[j] = (word[2 * j] >> 16) | (word[2 * j + 1] & 0xffff0000u);
+                }
+                o[2 * t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&even), p, o[2 * t], 0, 0, 0);
+                o[2 * t + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&odd), p, o[2 * t + 1], 0, 0, 0);
+            }
+        }
+    }
+    weight += __shfl_xor(weight, 32, WAVE);
+    if (!pair_valid) return;
+    const size_t item = (size_t)row * n_heads + head;
+    if (n_runs == 1) {
+        float inverse;
+        if (sinks) {
+            const float sink = sinks[head], highest = fmaxf(top, sink);
+            const float shrink = expf(top - highest);
+            inverse = shrink / (weight * shrink + expf(sink - highest));
+        } else {
+            inverse = 1.0f / weight;
+        }
+        float* out_row = out + item * R;
+#pragma unroll
+        for (int i = 0; i < RT; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int d = 64 * (i / 2) + 2 * (8 * (v / 4) + 4 * half + (v % 4)) + (i % 2);
+                if (d < R) out_row[d] = o[i][v] * inverse;
+            }
+        return;
+    }
+    float* mine = parts + (item * n_runs + run) * (R + 2);
+#pragma unroll
+    for (int i = 0; i < RT; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int d = 64 * (i / 2) + 2 * (8 * (v / 4) + 4 * half + (v % 4)) + (i % 2);
+            if (d < R) mine[d] = o[i][v];
+        }
+    if (half == 0) {
+        mine[R] = top;
+        mine[R + 1] = weight;
+    }
+}
+
+struct LatentMfmaArgs {
+    const float* q; const bf16_t* pages; const float* sinks; float* out; float* parts; const int* q_starts; const int* context_lens;
+    const int* block_tables; int max_blocks, n_heads, R, page_size; float scale; int run_length; dim3 grid; hipStream_t stream;
+};
+
+template <int DK, int RT>
+void launch_latent_mfma(const LatentMfmaArgs& a) {
+    latent_attention_mfma_kernel<DK, RT><<<a.grid, 64, 0, a.stream>>>(a.q, a.pages, a.sinks, a.out, a.parts, a.q_starts, a.context_lens, a.block_tables,
+                                                                      a.max_blocks, a.n_heads, a.R, a.page_size, a.scale, a.run_length);
+}
+
+template <int DK>
+bool launch_latent_mfma_rt(const LatentMfmaArgs& a) {
+    if (a.R <= 64) launch_latent_mfma<DK, 2>(a);
+    else if constexpr (DK >= 6) {
+        if (a.R <= 128) launch_latent_mfma<DK, 4>(a);
+        else if constexpr (DK >= 12) launch_latent_mfma<DK, 8>(a);
+        else return false;
+    } else return false;
+    return true;
+}
+
 template <typename KernelT>
 int allow_lds(KernelT kernel, size_t bytes, const char* what) {
     if (bytes <= 48 * 1024) return 0;
@@ -411,6 +579,51 @@ MLLM_API int mllm_latent_attention(const float* q, const void* pages, const floa
     if (dtype == MLLM_F32) launch_latent_hg<float>(args);
     else launch_latent_hg<bf16_t>(args);
     int status = mllm_check_launch("latent_attention");
+    if (status || n_runs == 1) return status;
+    const long long items = (long long)n_rows * n_heads;
+    mllm_count_kernel(MLLM_K_LATENT_MERGE);
+    latent_merge_kernel<<<(int)((items + 3) / 4), 256, 0, stream>>>(parts, sinks, token_request, out, n_rows, n_heads, n_runs, R);
+    return mllm_check_launch("latent_merge");
+}
+
+// Rows of how many elements the matrix-core kernel takes: the smallest such size that holds `needed` elements (0: none does,
+// and the rows are walked by the kernel above, which takes any multiple of 16 bytes).
+MLLM_API int mllm_latent_mfma_row_size(int needed) {
+    for (int size : {32, 64, 96, 128, 192, 288})
+        if (needed <= size) return size;
+    return 0;
+}
+
+MLLM_API int mllm_latent_attention_mfma_supported(int R, int D, int dtype) {
+    return dtype == MLLM_BF16 && R > 0 && R <= D && R <= 256 && mllm_latent_mfma_row_size(D) == D;
+}
+
+// q_starts [requests + 1] and context_lens [requests] (negative: a padding request): each request's rows are consecutive, its
+// first row's position is its stored length. max_pairs: the most (token, head) pairs any request brings.
+MLLM_API int mllm_latent_attention_mfma(const float* q, const void* pages, const float* sinks, float* out, float* parts, const int* token_request,
+                                        const int* q_starts, const int* context_lens, const int* block_tables, int max_blocks, int n_rows,
+                                        int n_requests, int max_pairs, int n_heads, int R, int D, int page_size, float scale, int n_runs,
+                                        int run_length, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && n_requests >= 0 && n_heads > 0 && max_blocks > 0 && page_size > 0 && max_pairs > 0, "latent_attention_mfma: bad sizes");
+    MLLM_REQUIRE(mllm_latent_attention_mfma_supported(R, D, MLLM_BF16), "latent_attention_mfma: no kernel for rows of %d elements with a latent of %d", D, R);
+    MLLM_REQUIRE(n_runs >= 1 && n_runs <= 65535 && n_requests <= 65535 && run_length >= 1 && (n_runs == 1 || run_length % 32 == 0), "latent_attention_mfma: bad runs");
+    MLLM_REQUIRE(n_runs == 1 || parts != nullptr, "latent_attention_mfma: runs need room for their sums");
+    if (n_rows == 0 || n_requests == 0) return 0;
+    if (n_runs == 1) run_length = 1 << 30;
+    LatentMfmaArgs a{q, (const bf16_t*)pages, sinks, out, parts, q_starts, context_lens, block_tables, max_blocks, n_heads, R, page_size, scale, run_length,
+                     dim3(ceil_div(max_pairs, 32), n_requests, n_runs), stream};
+    mllm_count_kernel(MLLM_K_LATENT_ATTENTION);
+    bool launched = false;
+    switch (D / 16) {
+        case 2: launched = launch_latent_mfma_rt<2>(a); break;
+        case 4: launched = launch_latent_mfma_rt<4>(a); break;
+        case 6: launched = launch_latent_mfma_rt<6>(a); break;
+        case 8: launched = launch_latent_mfma_rt<8>(a); break;
+        case 12: launched = launch_latent_mfma_rt<12>(a); break;
+        case 18: launched = launch_latent_mfma_rt<18>(a); break;
+    }
+    MLLM_REQUIRE(launched, "latent_attention_mfma: no kernel for rows of %d elements with a latent of %d", D, R);
+    int status = mllm_check_launch("latent_attention_mfma");
     if (status || n_runs == 1) return status;
     const long long items = (long long)n_rows * n_heads;
     mllm_count_kernel(MLLM_K_LATENT_MERGE);

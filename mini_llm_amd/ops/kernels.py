@@ -931,11 +931,22 @@ def latent_attention_supported(rank: int, row_size: int, dtype) -> bool:
     return bool(library().mllm_latent_attention_supported(int(rank), int(row_size), _code(dtype)))
 
 
-def latent_attention(q_full, pages, sinks, token_request, positions, block_tables, rank, scale, max_len=None):
+def latent_row_size(needed: int) -> int:
+    """The size of a cached row that holds ``needed`` elements: one the matrix-core kernel takes where there is one, else the
+    next multiple of 8 (whole 16-byte pieces in either precision). What lies beyond the needed elements is zero."""
+    size = int(library().mllm_latent_mfma_row_size(int(needed)))
+    return size if size else -(-int(needed) // 8) * 8
+
+
+def latent_attention(q_full, pages, sinks, token_request, positions, block_tables, rank, scale, max_len=None, q_starts=None, context_lens=None,
+                     max_q_len=None):
     """Causal attention of each row's heads over its request's cached rows: score = scale * q_full[row, h] . cached row, softmax
     with exp(sinks[h]) in the denominator (``sinks`` None: without), the sum taken over the rows' first ``rank`` elements.
     q_full: float32 [rows, n_heads, row_size]; pages [num_pages, 1, page_size, row_size]. Returns float32 [rows, n_heads,
-    rank]. Few rows with many keys are cut into runs of keys, a block each (``max_len``: the longest sequence of the batch)."""
+    rank]. Few rows with many keys are cut into runs of keys (``max_len``: the longest sequence of the batch).
+    With ``q_starts`` ([requests + 1]: each request's rows are consecutive), ``context_lens`` ([requests]: the position of a
+    request's first row; negative: a padding request) and ``max_q_len``, a bfloat16 cache of a row size the matrix-core kernel
+    takes runs through that kernel (32 (token, head) pairs of a request to a wave)."""
     _device_tensor(q_full, "q_full", torch.float32, 3)
     _device_tensor(pages, "pages", dim=4)
     n, n_heads, row_size = q_full.shape
@@ -951,8 +962,26 @@ def latent_attention(q_full, pages, sinks, token_request, positions, block_table
     out = torch.empty((n, n_heads, rank), dtype=torch.float32, device=q_full.device)
     if n == 0:
         return out
+    lib = library()
     reach = block_tables.shape[1] * page_size
     longest = reach if max_len is None else max(1, min(int(max_len), reach))
+    if (q_starts is not None and context_lens is not None and max_q_len is not None
+            and lib.mllm_latent_attention_mfma_supported(int(rank), row_size, _code(pages.dtype))):
+        _device_tensor(q_starts, "q_starts", torch.int32, 1)
+        _device_tensor(context_lens, "context_lens", torch.int32, 1)
+        n_requests = context_lens.shape[0]
+        _require(q_starts.shape[0] == n_requests + 1 and block_tables.shape[0] >= n_requests, "q_starts, context_lens and block tables do not match")
+        max_pairs = max(1, min(int(max_q_len), n)) * n_heads
+        waves = n_requests * -(-max_pairs // 32)
+        n_runs = max(1, min(LATENT_TARGET_WAVES // 2 // waves, longest // LATENT_RUN_MIN, 256))
+        run_length = -(-(-(-longest // n_runs)) // 64) * 64 if n_runs > 1 else reach
+        parts = torch.empty((n, n_heads, n_runs, rank + 2), dtype=torch.float32, device=q_full.device) if n_runs > 1 else None
+        if n_runs == 1:   # rows that belong to no request (padding) are reached by no wave; with runs the merge writes every row
+            out.zero_()
+        check(lib.mllm_latent_attention_mfma(_ptr(q_full), _ptr(pages), _ptr(sinks), _ptr(out), _ptr(parts), _ptr(token_request), _ptr(q_starts),
+                                             _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n, n_requests, max_pairs, n_heads,
+                                             int(rank), row_size, page_size, float(scale), n_runs, run_length, _stream()))
+        return out
     # a wave takes a row's keys for a group of heads: few rows with many keys are cut into runs, a wave each
     waves = n * -(-n_heads // int(library().mllm_latent_attention_head_group(n_heads)))
     n_runs = max(1, min(LATENT_TARGET_WAVES // waves, longest // LATENT_RUN_MIN, 256))

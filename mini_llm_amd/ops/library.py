@@ -54,6 +54,9 @@ _SIGNATURES = {
     "mllm_heads_linear": [P, c_int, c_int, c_int, P, c_int, P, c_int, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_latent_attention_supported": [c_int, c_int, c_int],
     "mllm_latent_attention_head_group": [c_int],
+    "mllm_latent_mfma_row_size": [c_int],
+    "mllm_latent_attention_mfma_supported": [c_int, c_int, c_int],
+    "mllm_latent_attention_mfma": [P, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
     "mllm_latent_attention": [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
 }
 

@@ -30,8 +30,8 @@ class LatentAttention(Mixer):
         self.width, self.n_heads, self.dim, self.rot_dim, self.vdim, self.kv_rank = width, n_heads, dim, rot_dim, vdim, kv_rank
         self.scale, self.eps, self.rotary = float(scale), float(eps), rotary
         self.has_sink, self.gated, self.own_latent = sink, gated, own_latent
-        # a cached row: [latent | rotated key part | zeros up to a multiple of 32 bytes] (whole 16-byte pieces in either precision)
-        self.row_size = -(-(kv_rank + rot_dim) // 8) * 8
+        # a cached row: [latent | rotated key part | zeros up to a size the attention kernels take]
+        self.row_size = kernels.latent_row_size(kv_rank + rot_dim)
         self.w_in = self.uk_t = self.uv = self.o = self.sink = self.dkv_norm = None
 
     def tensor_specs(self):
@@ -79,8 +79,10 @@ class LatentAttention(Mixer):
         q_full = kernels.latent_rows(q, dkv, self.dkv_norm, self.eps, self.rotary.frequencies(x.device), self.rotary.magnitude, self.rotary.dims,
                                      batch.positions, ctx.group.slots, ctx.k_pages, H, self.dim, self.rot_dim, self.kv_rank)
         kernels.heads_linear(q, self.uk_t, q_full, n_heads=H, k=self.dim, x_head_stride=self.dim + self.rot_dim)
+        whole = getattr(batch, "first_row", 0) == 0   # a part of a batch numbers its rows from the whole batch's top
         summed = kernels.latent_attention(q_full, ctx.k_pages, self.sink, batch.token_request, batch.positions, ctx.group.block_tables,
-                                          self.kv_rank, self.scale, max_len=batch.max_total_len)
+                                          self.kv_rank, self.scale, max_len=batch.max_total_len, q_starts=batch.q_starts if whole else None,
+                                          context_lens=batch.context_lens, max_q_len=batch.max_q_len)
         mixed = torch.empty((rows, H, self.vdim), dtype=x.dtype, device=x.device)
         kernels.heads_linear(summed, self.uv, mixed, n_heads=H, k=self.kv_rank, x_head_stride=self.kv_rank, gate=gate)
         return kernels.linear(mixed.view(rows, H * self.vdim), self.o, residual=residual, out_dtype=torch.float32)

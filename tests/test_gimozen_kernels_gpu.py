@@ -129,7 +129,7 @@ def test_latent_rows_rotate_and_keep(dtype, heads, dim, rot, rot_dims, rank):
     rot_config = {"dims": rot_dims, "base": 100.0, "scaling": {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 1.0}}
     part = RotaryEncoding(rot_dims, 100.0, rot_config["scaling"])
     rows, page_size, n_pages, eps = 6, 4, 4, 1e-5
-    row_size = -(-(rank + rot) // 8) * 8
+    row_size = k.latent_row_size(rank + rot)
     positions = np.array([0, 1, 5, 37, 300, 1021])
     slots = np.array([3, -1, 0, 9, 14, 6])
     q = rounded(rng.normal(0, 1, (rows, heads * (dim + rot))), dtype)
@@ -182,7 +182,7 @@ def test_heads_linear(w_dtype, rows, heads, n, k_size):
 def latent_case(rng, dtype, lengths, heads, rank, rot, page_size, sharp=None):
     """Requests of the given lengths, their cached rows spread over shuffled pages; one query row per request at its last
     position (decode) and, for the first request, a query at every position (a portion)."""
-    row_size = -(-(rank + rot) // 8) * 8
+    row_size = kernels().latent_row_size(rank + rot)
     n_blocks = [-(-n // page_size) for n in lengths]
     order = rng.permutation(sum(n_blocks) + 3)
     pages = torch.zeros((len(order), 1, page_size, row_size), dtype=dtype)
@@ -201,12 +201,22 @@ def latent_case(rng, dtype, lengths, heads, rank, rot, page_size, sharp=None):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("by_request", [False, True])
 @pytest.mark.parametrize("heads,rank,rot,page_size,lengths", [(3, 40, 8, 16, [70, 1, 33, 16, 17]), (17, 64, 32, 64, [200, 64, 65]), (1, 21, 16, 4, [9, 700]),
-                                                             (2, 300, 20, 32, [130, 31])])
-def test_latent_attention_with_a_sink(dtype, heads, rank, rot, page_size, lengths):
+                                                             (2, 300, 20, 32, [130, 31]), (12, 256, 32, 64, [100, 300]), (5, 130, 8, 32, [40, 41, 90])])
+def test_latent_attention_with_a_sink(dtype, heads, rank, rot, page_size, lengths, by_request):
+    # by_request: the batch's requests are named too (first rows, stored lengths), which lets a bfloat16 cache of a fitting row
+    # size run on the matrix cores (queries and weights rounded to bfloat16 there)
     k = kernels()
     rng = np.random.default_rng(rank + heads)
     pages, tables, cached, row_size = latent_case(rng, dtype, lengths, heads, rank, rot, page_size)
+    extra = {}
+    if by_request:
+        starts = [0, lengths[0]] + [lengths[0] + i for i in range(1, len(lengths))]
+        extra = dict(q_starts=torch.tensor(starts, dtype=torch.int32).cuda(), context_lens=torch.tensor([0] + [n - 1 for n in lengths[1:]], dtype=torch.int32).cuda(),
+                     max_q_len=lengths[0])
+    on_matrix_cores = by_request and dtype == torch.bfloat16 and bool(k.library().mllm_latent_attention_mfma_supported(rank, row_size, 1))
+    bound = dict(atol=3e-2, rtol=3e-2) if on_matrix_cores else dict(atol=2e-5, rtol=2e-4)
     # rows: every position of request 0 (a whole prompt), then the last position of the others
     token_request = [0] * lengths[0] + list(range(1, len(lengths)))
     positions = list(range(lengths[0])) + [n - 1 for n in lengths[1:]]
@@ -217,13 +227,13 @@ def test_latent_attention_with_a_sink(dtype, heads, rank, rot, page_size, length
     for use_sink in (True, False):
         for max_len in (None, max(lengths)):
             got = k.latent_attention(gpu(q), pages, gpu(sinks) if use_sink else None, torch.tensor(token_request, dtype=torch.int32).cuda(),
-                                     torch.tensor(positions, dtype=torch.int32).cuda(), torch.tensor(tables).cuda(), rank, scale, max_len=max_len).cpu().numpy()
+                                     torch.tensor(positions, dtype=torch.int32).cuda(), torch.tensor(tables).cuda(), rank, scale, max_len=max_len, **extra).cpu().numpy()
             for row, (request, position) in enumerate(zip(token_request, positions)):
                 keys = cached[request][: position + 1]
                 for head in range(heads):
                     scores = (keys @ q[row, head])[None, :] * scale
                     weights = plain.softmax_rows(scores, np.ones_like(scores, dtype=bool), sink=float(sinks[head]) if use_sink else None)
-                    np.testing.assert_allclose(got[row, head], (weights @ keys[:, :rank])[0], atol=2e-5, rtol=2e-4,
+                    np.testing.assert_allclose(got[row, head], (weights @ keys[:, :rank])[0], **bound,
                                                err_msg=f"row {row} (request {request}, position {position}) head {head} sink {use_sink}")
 
 
