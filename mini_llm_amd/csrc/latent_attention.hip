@@ -96,6 +96,54 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const void* __restric
     }
 }
 
+// The same products on the matrix cores, for bfloat16 matrices with K a multiple of 16 and x rows that start on 16-byte
+// boundaries: out^T tile [32 columns, 32 rows] = W_h tile . x_h tile^T, a wave a tile, both operands as they lie in memory (a
+// lane's 16-byte piece of its W row, and of its x row: eight bfloat16, or eight floats rounded to bfloat16 on the way).
+// The four waves of a block take four neighbouring column tiles of the same rows.
+template <typename XT>
+__global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const XT* __restrict__ x, int x_row_stride, int x_head_stride,
+                                                                const bf16_t* __restrict__ w, const void* __restrict__ gate, int gate_code,
+                                                                int gate_row_stride, void* __restrict__ out, int out_code, int out_row_stride,
+                                                                int out_head_stride, int n_rows, int N, int K) {
+    const int lane = threadIdx.x % WAVE, lane32 = lane % 32, half = lane / 32;
+    const int head = blockIdx.y, row0 = blockIdx.x * 32;
+    const int n0 = (blockIdx.z * 4 + threadIdx.x / WAVE) * 32;
+    if (n0 >= N) return;
+    const bf16_t* w_row = w + ((size_t)head * N + min(n0 + lane32, N - 1)) * K + 8 * half;
+    const XT* x_row = x + (size_t)min(row0 + lane32, n_rows - 1) * x_row_stride + (size_t)head * x_head_stride + 8 * half;
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+    for (int k = 0; k < K; k += 16) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(w_row + k);
+        bf16x8 b;
+        if constexpr (sizeof(XT) == 2) {
+            b = *reinterpret_cast<const bf16x8*>(x_row + k);
+        } else {
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(x_row + k), hi = *reinterpret_cast<const f32x4*>(x_row + k + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                b[e] = static_cast<bf16_t>(lo[e]);
+                b[4 + e] = static_cast<bf16_t>(hi[e]);
+            }
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+    }
+    const int row = row0 + lane32;
+    if (row >= n_rows) return;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const int n = n0 + 8 * (v / 4) + 4 * half + (v % 4);
+        if (n >= N) continue;
+        float value = acc[v];
+        if (gate) {
+            const float g = load_as_float(gate, (size_t)row * gate_row_stride + (size_t)head * N + n, gate_code);
+            value *= 1.0f / (1.0f + expf(-g));
+        }
+        store_from_float(out, (size_t)row * out_row_stride + (size_t)head * out_head_stride + n, out_code, value);
+    }
+}
+
 constexpr int LATENT_ROWS = 4;   // rows of the batch a block takes, a wave each
 
 template <typename T>
@@ -541,8 +589,20 @@ MLLM_API int mllm_heads_linear(const void* x, int x_dtype, int x_row_stride, int
     const size_t lds = ((size_t)HEADS_ROWS * K + (size_t)(threads / cols - 1) * cols * HEADS_ROWS) * sizeof(float);
     MLLM_REQUIRE(lds <= 64 * 1024, "heads_linear: K = %d is more than a block holds in LDS", K);
     if (n_rows == 0) return 0;
-    dim3 grid(ceil_div(n_rows, HEADS_ROWS), n_heads);
     mllm_count_kernel(MLLM_K_HEADS_LINEAR);
+    const size_t x_element = x_dtype == MLLM_F32 ? 4 : 2;
+    if (w_dtype == MLLM_BF16 && K % 16 == 0 && (size_t)x % 16 == 0 && (x_row_stride * x_element) % 16 == 0 && (x_head_stride * x_element) % 16 == 0 &&
+        (size_t)w % 16 == 0) {
+        dim3 tiles(ceil_div(n_rows, 32), n_heads, ceil_div(N, 128));
+        if (x_dtype == MLLM_F32)
+            heads_linear_mfma_kernel<float><<<tiles, 256, 0, stream>>>((const float*)x, x_row_stride, x_head_stride, (const bf16_t*)w, gate, gate_dtype,
+                                                                       gate_row_stride, out, out_dtype, out_row_stride, out_head_stride, n_rows, N, K);
+        else
+            heads_linear_mfma_kernel<bf16_t><<<tiles, 256, 0, stream>>>((const bf16_t*)x, x_row_stride, x_head_stride, (const bf16_t*)w, gate, gate_dtype,
+                                                                        gate_row_stride, out, out_dtype, out_row_stride, out_head_stride, n_rows, N, K);
+        return mllm_check_launch("heads_linear");
+    }
+    dim3 grid(ceil_div(n_rows, HEADS_ROWS), n_heads);
     if (w_dtype == MLLM_F32) {
         if (allow_lds(heads_linear_kernel<float>, lds, "heads_linear")) return 1;
         heads_linear_kernel<float><<<grid, threads, lds, stream>>>(x, x_dtype, x_row_stride, x_head_stride, (const float*)w, gate, gate_dtype, gate_row_stride, out, out_dtype,

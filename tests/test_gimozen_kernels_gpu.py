@@ -161,22 +161,29 @@ def test_latent_rows_rotate_and_keep(dtype, heads, dim, rot, rot_dims, rank):
 
 
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("rows,heads,n,k_size", [(1, 3, 40, 16), (17, 2, 24, 64), (33, 1, 300, 21), (5, 5, 7, 512)])
-def test_heads_linear(w_dtype, rows, heads, n, k_size):
+@pytest.mark.parametrize("gap", [3, 16])
+@pytest.mark.parametrize("rows,heads,n,k_size", [(1, 3, 40, 16), (17, 2, 24, 64), (33, 1, 300, 21), (5, 5, 7, 512), (70, 3, 130, 32)])
+def test_heads_linear(w_dtype, rows, heads, n, k_size, gap):
+    # gap: how far the heads of x lie apart beyond their K elements. With a gap of 16 the rows start on 16-byte boundaries, and
+    # bfloat16 matrices with K a multiple of 16 then run on the matrix cores, where x is rounded to bfloat16 on its way in
     k = kernels()
     rng = np.random.default_rng(rows)
-    x = rng.normal(0, 1, (rows, heads, k_size + 3))   # heads lie further apart than their K elements
+    x = rng.normal(0, 1, (rows, heads, k_size + gap))
     w = rounded(rng.normal(0, 1, (heads, n, k_size)), w_dtype)
     gate = rng.normal(0, 2, (rows, heads * n))
+    rounds_x = w_dtype == torch.bfloat16 and gap == 16 and k_size % 16 == 0
+    bound = dict(atol=0.02 * k_size ** 0.5, rtol=2e-2) if rounds_x else dict(atol=1e-4, rtol=1e-4)
     out = torch.full((rows, heads, n + 2), 5.0, dtype=torch.float32).cuda()
-    k.heads_linear(gpu(x).view(rows, -1), gpu(w, w_dtype), out, n_heads=heads, k=k_size, x_head_stride=k_size + 3, gate=gpu(gate))
+    k.heads_linear(gpu(x).view(rows, -1), gpu(w, w_dtype), out, n_heads=heads, k=k_size, x_head_stride=k_size + gap, gate=gpu(gate))
     want = np.einsum("rhk,hnk->rhn", x[:, :, :k_size], w) * plain.sigmoid(gate.reshape(rows, heads, n))
     got = out.cpu().numpy()
-    np.testing.assert_allclose(got[:, :, :n], want, atol=1e-4, rtol=1e-4)
+    np.testing.assert_allclose(got[:, :, :n], want, **bound)
     assert (got[:, :, n:] == 5).all()
+    # x in bfloat16 (exact on either path), the result in bfloat16
+    x16 = rounded(x, torch.bfloat16)
     out16 = torch.zeros((rows, heads, n), dtype=torch.bfloat16).cuda()
-    k.heads_linear(gpu(x).view(rows, -1), gpu(w, w_dtype), out16, n_heads=heads, k=k_size, x_head_stride=k_size + 3)
-    np.testing.assert_allclose(out16.float().cpu().numpy(), np.einsum("rhk,hnk->rhn", x[:, :, :k_size], w), atol=0.1, rtol=1e-2)
+    k.heads_linear(gpu(x16, torch.bfloat16).view(rows, -1), gpu(w, w_dtype), out16, n_heads=heads, k=k_size, x_head_stride=k_size + gap)
+    np.testing.assert_allclose(out16.float().cpu().numpy(), np.einsum("rhk,hnk->rhn", x16[:, :, :k_size], w), atol=0.1, rtol=1e-2)
 
 
 def latent_case(rng, dtype, lengths, heads, rank, rot, page_size, sharp=None):
