@@ -114,6 +114,7 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const XT* __rest
     f32x16 acc;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+#pragma unroll 4
     for (int k = 0; k < K; k += 16) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(w_row + k);
         bf16x8 b;
@@ -313,48 +314,52 @@ __global__ __launch_bounds__(64 * LATENT_ROWS) void latent_attention_kernel(
     }
 }
 
-// out[row, head] = sum_p o_p e^(m_p - M) / (sum_p l_p e^(m_p - M) + e^(sink - M)) over the runs of a (row, head); a wave each.
-// Lane p takes run p's maximum and weight (and the next 64 runs' after them), so the statistics cost one trip to memory; the
-// sums over the runs are taken four loads at a time.
+// out[row, head] = sum_p o_p e^(m_p - M) / (sum_p l_p e^(m_p - M) + e^(sink - M)) over the runs of a (row, head); a block each.
+// Thread p takes run p's maximum and weight into LDS (one trip to memory for all of them), every thread then knows M and the
+// denominator, takes an element of the latent and adds up its runs, eight loads under way at a time.
+constexpr int MERGE_MAX_RUNS = 256;
+
 __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ parts, const float* __restrict__ sinks,
                                                            const int* __restrict__ token_request, float* __restrict__ out, int n_rows,
                                                            int n_heads, int n_runs, int R) {
-    const int lane = threadIdx.x % WAVE;
-    const long long item = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (item >= (long long)n_rows * n_heads) return;
-    const int token = (int)(item / n_heads), head = (int)(item % n_heads);
+    __shared__ float factor[MERGE_MAX_RUNS];
+    __shared__ float inverse_total;
+    const int item = blockIdx.x, token = item / n_heads, head = item % n_heads;
     float* out_row = out + (size_t)item * R;
-    if (token_request[token] < 0) {
-        for (int d = lane; d < R; d += WAVE) out_row[d] = 0.0f;
+    if (token_request[token] < 0) {   // uniform over the block
+        for (int d = threadIdx.x; d < R; d += blockDim.x) out_row[d] = 0.0f;
         return;
     }
     const float* runs = parts + (size_t)item * n_runs * (R + 2);
+    const int p = threadIdx.x;
+    const float my_top = p < n_runs ? runs[(size_t)p * (R + 2) + R] : -INFINITY;
+    const float my_weight = p < n_runs ? runs[(size_t)p * (R + 2) + R + 1] : 0.0f;
+    factor[p] = my_top;
+    __syncthreads();
     const float sink = sinks ? sinks[head] : -INFINITY;
-    float my_top = -INFINITY;
-    for (int p = lane; p < n_runs; p += WAVE) my_top = fmaxf(my_top, runs[(size_t)p * (R + 2) + R]);
-    const float top = fmaxf(sink, wave_max_total(my_top));   // finite: the first run always holds a key
-    float my_total = 0.0f;
-    for (int p = lane; p < n_runs; p += WAVE) {
-        const float m = runs[(size_t)p * (R + 2) + R];
-        my_total += m == -INFINITY ? 0.0f : runs[(size_t)p * (R + 2) + R + 1] * expf(m - top);
-    }
-    const float total = wave_total(my_total) + (sinks ? expf(sink - top) : 0.0f);
-    const float inverse = 1.0f / total;
-    for (int d0 = 0; d0 < R; d0 += WAVE) {
-        const int d = min(d0 + lane, R - 1);
+    float top = sink;
+    for (int other = 0; other < n_runs; other++) top = fmaxf(top, factor[other]);   // finite: the first run always holds a key
+    __syncthreads();
+    const float mine = my_top == -INFINITY ? 0.0f : expf(my_top - top);
+    factor[p] = mine;
+    // the denominator: every wave adds up its runs' shares, the first wave the waves'
+    __shared__ float wave_share[4];
+    const float share = wave_total(mine * my_weight);
+    if (threadIdx.x % WAVE == 0) wave_share[threadIdx.x / WAVE] = share;
+    __syncthreads();
+    if (threadIdx.x == 0) inverse_total = 1.0f / (wave_share[0] + wave_share[1] + wave_share[2] + wave_share[3] + (sinks ? expf(sink - top) : 0.0f));
+    __syncthreads();
+    const float inverse = inverse_total;
+    for (int d = threadIdx.x; d < R; d += blockDim.x) {
         float sum = 0.0f;
-        for (int p0 = 0; p0 < n_runs; p0 += 4) {
-            float o[4], m[4];
+        for (int p0 = 0; p0 < n_runs; p0 += 8) {
+            float o[8];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const size_t at = (size_t)min(p0 + u, n_runs - 1) * (R + 2);
-                o[u] = runs[at + d];
-                m[u] = runs[at + R];
-            }
+            for (int u = 0; u < 8; u++) o[u] = runs[(size_t)min(p0 + u, n_runs - 1) * (R + 2) + d];
 #pragma unroll
-            for (int u = 0; u < 4; u++) sum += p0 + u < n_runs && m[u] != -INFINITY ? o[u] * expf(m[u] - top) : 0.0f;
+            for (int u = 0; u < 8; u++) sum += p0 + u < n_runs ? o[u] * factor[p0 + u] : 0.0f;
         }
-        if (d0 + lane < R) out_row[d] = sum * inverse;
+        out_row[d] = sum * inverse;
     }
 }
 
@@ -630,7 +635,7 @@ MLLM_API int mllm_latent_attention(const float* q, const void* pages, const floa
     MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && max_blocks > 0 && page_size > 0, "latent_attention: bad sizes");
     MLLM_REQUIRE(dtype == MLLM_F32 || dtype == MLLM_BF16, "latent_attention: unknown dtype %d", dtype);
     MLLM_REQUIRE(mllm_latent_attention_supported(R, D, dtype), "latent_attention: no kernel for rows of %d elements with a latent of %d", D, R);
-    MLLM_REQUIRE(n_runs >= 1 && n_runs <= 65535 && run_length >= 1, "latent_attention: bad runs");
+    MLLM_REQUIRE(n_runs >= 1 && n_runs <= MERGE_MAX_RUNS && run_length >= 1, "latent_attention: bad runs");
     MLLM_REQUIRE(n_runs == 1 || parts != nullptr, "latent_attention: runs need room for their sums");
     if (n_rows == 0) return 0;
     if (n_runs == 1) run_length = 1 << 30;
@@ -642,7 +647,7 @@ MLLM_API int mllm_latent_attention(const float* q, const void* pages, const floa
     if (status || n_runs == 1) return status;
     const long long items = (long long)n_rows * n_heads;
     mllm_count_kernel(MLLM_K_LATENT_MERGE);
-    latent_merge_kernel<<<(int)((items + 3) / 4), 256, 0, stream>>>(parts, sinks, token_request, out, n_rows, n_heads, n_runs, R);
+    latent_merge_kernel<<<(int)items, 256, 0, stream>>>(parts, sinks, token_request, out, n_rows, n_heads, n_runs, R);
     return mllm_check_launch("latent_merge");
 }
 
@@ -666,7 +671,7 @@ MLLM_API int mllm_latent_attention_mfma(const float* q, const void* pages, const
                                         int run_length, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_requests >= 0 && n_heads > 0 && max_blocks > 0 && page_size > 0 && max_pairs > 0, "latent_attention_mfma: bad sizes");
     MLLM_REQUIRE(mllm_latent_attention_mfma_supported(R, D, MLLM_BF16), "latent_attention_mfma: no kernel for rows of %d elements with a latent of %d", D, R);
-    MLLM_REQUIRE(n_runs >= 1 && n_runs <= 65535 && n_requests <= 65535 && run_length >= 1 && (n_runs == 1 || run_length % 32 == 0), "latent_attention_mfma: bad runs");
+    MLLM_REQUIRE(n_runs >= 1 && n_runs <= MERGE_MAX_RUNS && n_requests <= 65535 && run_length >= 1 && (n_runs == 1 || run_length % 32 == 0), "latent_attention_mfma: bad runs");
     MLLM_REQUIRE(n_runs == 1 || parts != nullptr, "latent_attention_mfma: runs need room for their sums");
     if (n_rows == 0 || n_requests == 0) return 0;
     if (n_runs == 1) run_length = 1 << 30;
@@ -687,6 +692,6 @@ MLLM_API int mllm_latent_attention_mfma(const float* q, const void* pages, const
     if (status || n_runs == 1) return status;
     const long long items = (long long)n_rows * n_heads;
     mllm_count_kernel(MLLM_K_LATENT_MERGE);
-    latent_merge_kernel<<<(int)((items + 3) / 4), 256, 0, stream>>>(parts, sinks, token_request, out, n_rows, n_heads, n_runs, R);
+    latent_merge_kernel<<<(int)items, 256, 0, stream>>>(parts, sinks, token_request, out, n_rows, n_heads, n_runs, R);
     return mllm_check_launch("latent_merge");
 }

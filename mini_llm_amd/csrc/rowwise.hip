@@ -141,6 +141,61 @@ __global__ __launch_bounds__(256) void head_norm_kernel(const T* __restrict__ qk
     }
 }
 
+// The same for heads whose sizes are whole 16-byte pieces: LPH lanes take a head, a piece each (LPH a power of two, LPH pieces
+// hold head_size elements), so a wave takes 64 / LPH heads and every lane moves 16 bytes in and 16 bytes out.
+template <typename T, int LPH>
+__global__ __launch_bounds__(256) void head_norm_pieces_kernel(const T* __restrict__ qkv, int qkv_stride, const float* __restrict__ q_gain,
+                                                               const float* __restrict__ k_gain, float eps, float temp_coef, int temp_every,
+                                                               const int* __restrict__ positions, const int* __restrict__ slots,
+                                                               T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                               int n_rows, int n_heads, int n_kv_heads, int dim, int vdim, int head_size,
+                                                               int page_size, int write_cache) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const int per_row = n_heads + 2 * n_kv_heads;
+    const long long item = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / LPH;
+    const int at = (threadIdx.x % LPH) * VEC;   // the lane's first element of the head
+    const bool live = item < (long long)n_rows * per_row;
+    const int row = live ? (int)(item / per_row) : 0, head = live ? (int)(item % per_row) : 0;
+    const bool is_q = head < n_heads, is_k = !is_q && head < n_heads + n_kv_heads;
+    const int own = is_q || is_k ? dim : vdim;   // the head's own elements
+    const int g = is_q ? head : (is_k ? head - n_heads : head - n_heads - n_kv_heads);
+    const T* in = qkv + (size_t)row * qkv_stride + (is_q ? 0 : (is_k ? n_heads * dim : (n_heads + n_kv_heads) * dim)) + (size_t)g * own;
+    const bool has = live && at < own;
+    Vec16 piece = {};
+    if (has) piece = *reinterpret_cast<const Vec16*>(in + at);
+    const T* e = reinterpret_cast<const T*>(&piece);
+    float values[VEC], squares = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        values[j] = to_float(e[j]);
+        squares += values[j] * values[j];
+    }
+#pragma unroll
+    for (int step = 1; step < LPH; step *= 2) squares += __shfl_xor(squares, step, WAVE);
+    if (!live || at >= head_size) return;
+    const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+    float factor = gain ? 1.0f / sqrtf(squares / (float)dim + eps) : 1.0f;
+    if (is_q && temp_coef != 0.0f) factor *= 1.0f + temp_coef * logf((float)((positions[row] + 1) / temp_every) + 1.0f);
+    T* out;
+    if (is_q) {
+        out = q_out + ((size_t)row * n_heads + head) * head_size;
+    } else {
+        if (!write_cache) return;
+        const int slot = slots[row];
+        if (slot < 0) return;
+        out = (is_k ? k_pages : v_pages) + (((size_t)(slot / page_size) * n_kv_heads + g) * page_size + slot % page_size) * head_size;
+    }
+    Vec16 result;
+    T* r = reinterpret_cast<T*>(&result);
+    if (is_q || is_k) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) r[j] = from_float<T>(has ? values[j] * factor * (gain ? gain[at + j] : 1.0f) : 0.0f);
+    } else {
+        result = piece;   // a value head as it is (zeros beyond its own elements)
+    }
+    *reinterpret_cast<Vec16*>(out + at) = result;
+}
+
 // Rotation of `dims` elements in the "rotate half" pairing: element i pairs with i + dims / 2, and the pair (u, v) at
 // position p becomes (u c - v s, v c + u s) with c = cos(p f_i) m, s = sin(p f_i) m. The angle is a 32-bit product.
 __device__ __forceinline__ void rotated_pair(float u, float v, int position, float frequency, float magnitude, float& a, float& b) {
@@ -264,18 +319,36 @@ MLLM_API int mllm_head_norm(const void* qkv, int qkv_stride, const float* q_gain
     MLLM_REQUIRE(!write_cache || (slots != nullptr && k_pages != nullptr && v_pages != nullptr), "head_norm: a cache write needs slots and pages");
     if (n_rows == 0) return 0;
     const long long items = (long long)n_rows * (n_heads + 2 * n_kv_heads);
-    const int blocks = (int)((items + 3) / 4);
     mllm_count_kernel(MLLM_K_HEAD_NORM);
+    const int vec = dtype == MLLM_F32 ? 4 : 2 * 4;
+    const bool pieces = dim % vec == 0 && vdim % vec == 0 && head_size % vec == 0 && head_size / vec <= 64 && qkv_stride % vec == 0 &&
+                        (size_t)qkv % 16 == 0 && (size_t)q_out % 16 == 0 && (size_t)k_pages % 16 == 0 && (size_t)v_pages % 16 == 0;
+#define HEAD_NORM_ARGS(T) (const T*)qkv, qkv_stride, q_gain, k_gain, eps, temp_coef, temp_every, positions, slots, (T*)q_out, (T*)k_pages, (T*)v_pages, \
+                          n_rows, n_heads, n_kv_heads, dim, vdim, head_size, page_size, write_cache
+    if (pieces && (dtype == MLLM_F32 || dtype == MLLM_BF16)) {
+        int lanes = 1;
+        while (lanes * vec < head_size) lanes *= 2;
+        const int blocks = (int)((items * lanes + 255) / 256);
+#define HEAD_NORM_PIECES(LPH)                                                                                                   \
+    case LPH:                                                                                                                   \
+        if (dtype == MLLM_F32) head_norm_pieces_kernel<float, LPH><<<blocks, 256, 0, stream>>>(HEAD_NORM_ARGS(float));        \
+        else head_norm_pieces_kernel<bf16_t, LPH><<<blocks, 256, 0, stream>>>(HEAD_NORM_ARGS(bf16_t));                        \
+        break;
+        switch (lanes) {
+            HEAD_NORM_PIECES(1) HEAD_NORM_PIECES(2) HEAD_NORM_PIECES(4) HEAD_NORM_PIECES(8) HEAD_NORM_PIECES(16) HEAD_NORM_PIECES(32)
+            HEAD_NORM_PIECES(64)
+        }
+#undef HEAD_NORM_PIECES
+        return mllm_check_launch("head_norm");
+    }
+    const int blocks = (int)((items + 3) / 4);
     if (dtype == MLLM_F32)
-        head_norm_kernel<float><<<blocks, 256, 0, stream>>>((const float*)qkv, qkv_stride, q_gain, k_gain, eps, temp_coef, temp_every, positions, slots,
-                                                            (float*)q_out, (float*)k_pages, (float*)v_pages, n_rows, n_heads, n_kv_heads, dim, vdim,
-                                                            head_size, page_size, write_cache);
+        head_norm_kernel<float><<<blocks, 256, 0, stream>>>(HEAD_NORM_ARGS(float));
     else if (dtype == MLLM_BF16)
-        head_norm_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)qkv, qkv_stride, q_gain, k_gain, eps, temp_coef, temp_every, positions, slots,
-                                                             (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, n_rows, n_heads, n_kv_heads, dim, vdim,
-                                                             head_size, page_size, write_cache);
+        head_norm_kernel<bf16_t><<<blocks, 256, 0, stream>>>(HEAD_NORM_ARGS(bf16_t));
     else
         MLLM_REQUIRE(false, "head_norm: unknown dtype %d", dtype);
+#undef HEAD_NORM_ARGS
     return mllm_check_launch("head_norm");
 }
 

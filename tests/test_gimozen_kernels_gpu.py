@@ -65,7 +65,7 @@ def test_silu_mul(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("dim,vdim,heads,kv_heads", [(16, 16, 4, 2), (24, 8, 3, 3), (8, 40, 2, 1), (80, 80, 1, 1)])
+@pytest.mark.parametrize("dim,vdim,heads,kv_heads", [(16, 16, 4, 2), (24, 8, 3, 3), (8, 40, 2, 1), (80, 80, 1, 1), (64, 64, 12, 4), (12, 20, 2, 1), (10, 6, 3, 3)])
 def test_head_norm_writes_queries_keys_and_values(dtype, dim, vdim, heads, kv_heads):
     k = kernels()
     rng = np.random.default_rng(dim)
