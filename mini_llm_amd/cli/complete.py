@@ -22,6 +22,8 @@ def parse_args(argv=None) -> argparse.Namespace:
     parser.add_argument("--device", default="auto", choices=("auto", "cpu", "cuda"), help="Inference device")
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--seed", type=int, default=0, help="Seed of the sampler")
+    parser.add_argument("--max-length", type=int, default=4096, help="Longest sequence, prompt and continuation: needed for a model without a position "
+                        "limit of its own (the cache holds four of them), and narrows a model's own")
     parser.add_argument("--tokens", default=None, help="Prompt as comma-separated token ids; prints the continuation and exits")
     return parser.parse_args(argv)
 
@@ -52,7 +54,7 @@ def main(argv=None) -> int:
         return 2
     from ..engine.engine import Engine, EngineOptions
 
-    engine = Engine(args.model, EngineOptions(dtype=args.dtype, max_sessions=4))
+    engine = Engine(args.model, EngineOptions(dtype=args.dtype, max_sessions=4, max_length=args.max_length))
     tokenizer = load_tokenizer(args.model)
     eos = engine.config.eos_token_id
 

@@ -14,7 +14,9 @@ __device__ __forceinline__ void store_from_float(void* base, size_t index, int c
     else reinterpret_cast<bf16_t*>(base)[index] = static_cast<bf16_t>(value);
 }
 
-// out = h / sqrt(mean(h^2) + eps) * g with h = alpha * x (+ y) and g = weight or 1 + weight. A wave per output row; a row
+// out = h / sqrt(mean(h^2) + eps) * g with h = alpha * x (+ y) and g = weight or 1 + weight. y may be n_partials partial
+// products of a product cut along K ([n_partials, rows, width], 32-bit): their sum is taken here, in a fixed order.
+// A wave per output row; a row
 // of up to 64 * REGS elements stays in registers between the two passes, a longer one is read again. row_index, if
 // given, names the input row of each output row. The result goes to `stream` (32-bit, what the residual stream goes on
 // with) and / or `rows` (the element type the next product reads); either may be null.
@@ -22,7 +24,7 @@ template <int REGS>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const void* __restrict__ y, int y_code, float alpha,
                                                        const int* __restrict__ row_index, const float* __restrict__ weight, int one_plus,
                                                        float eps, float* __restrict__ stream, void* __restrict__ rows, int rows_code,
-                                                       int n_rows, int width) {
+                                                       int n_rows, int width, int n_partials, long long partial_stride) {
     const int lane = threadIdx.x % WAVE;
     const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (row >= n_rows) return;
@@ -42,6 +44,20 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
             if (y_code == MLLM_F32) {
 #pragma unroll
                 for (int r = 0; r < REGS; r++) added[r] = reinterpret_cast<const float*>(y)[in_at + min(lane + r * WAVE, width - 1)];
+                // further partial products, a few asked for at a time (beyond the last one: the last once more, not added)
+                constexpr int AHEAD = REGS <= 16 ? 4 : 2;
+                for (int p0 = 1; p0 < n_partials; p0 += AHEAD) {
+                    float more[AHEAD][REGS];
+#pragma unroll
+                    for (int u = 0; u < AHEAD; u++)
+#pragma unroll
+                        for (int r = 0; r < REGS; r++)
+                            more[u][r] = reinterpret_cast<const float*>(y)[min(p0 + u, n_partials - 1) * partial_stride + in_at + min(lane + r * WAVE, width - 1)];
+#pragma unroll
+                    for (int u = 0; u < AHEAD; u++)
+#pragma unroll
+                        for (int r = 0; r < REGS; r++) added[r] += p0 + u < n_partials ? more[u][r] : 0.0f;
+                }
             } else {
 #pragma unroll
                 for (int r = 0; r < REGS; r++) added[r] = to_float(reinterpret_cast<const bf16_t*>(y)[in_at + min(lane + r * WAVE, width - 1)]);
@@ -71,13 +87,13 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
         float squares = 0.0f;
         for (int i = lane; i < width; i += WAVE) {
             float h = alpha * x[in_at + i];
-            if (y) h += load_as_float(y, in_at + i, y_code);
+            for (int p = 0; y && p < n_partials; p++) h += load_as_float(y, p * partial_stride + in_at + i, y_code);
             squares += h * h;
         }
         const float inverse = 1.0f / sqrtf(wave_total(squares) / (float)width + eps);
         for (int i = lane; i < width; i += WAVE) {
             float h = alpha * x[in_at + i];
-            if (y) h += load_as_float(y, in_at + i, y_code);
+            for (int p = 0; y && p < n_partials; p++) h += load_as_float(y, p * partial_stride + in_at + i, y_code);
             const float value = h * inverse * (plus + weight[i]);
             if (stream) stream[out_at + i] = value;
             if (rows) store_from_float(rows, out_at + i, rows_code, value);
@@ -290,16 +306,19 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ bot
 }  // namespace
 
 MLLM_API int mllm_rms_norm(const float* x, const void* y, int y_dtype, float alpha, const int* row_index, const float* weight, int one_plus,
-                           float eps, float* stream_out, void* rows_out, int rows_dtype, int n_rows, int width, hipStream_t stream) {
+                           float eps, float* stream_out, void* rows_out, int rows_dtype, int n_rows, int width, int n_partials,
+                           long long partial_stride, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && width > 0, "rms_norm: bad sizes rows=%d width=%d", n_rows, width);
     MLLM_REQUIRE(x != nullptr && weight != nullptr && (stream_out != nullptr || rows_out != nullptr), "rms_norm: a missing operand");
     MLLM_REQUIRE(y == nullptr || y_dtype == MLLM_F32 || y_dtype == MLLM_BF16, "rms_norm: unknown element type of the addend");
     MLLM_REQUIRE(rows_out == nullptr || rows_dtype == MLLM_F32 || rows_dtype == MLLM_BF16, "rms_norm: unknown element type of the rows");
     MLLM_REQUIRE(y == nullptr || row_index == nullptr, "rms_norm: gathered rows take no addend");
+    MLLM_REQUIRE(n_partials >= 1 && (n_partials == 1 || (y != nullptr && y_dtype == MLLM_F32 && partial_stride >= (long long)n_rows * width)),
+                 "rms_norm: partial products are 32-bit and lie a whole matrix apart");
     if (n_rows == 0) return 0;
     const int waves = 4, blocks = ceil_div(n_rows, waves);
     mllm_count_kernel(MLLM_K_RMS_NORM);
-#define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width)
+#define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width, n_partials, partial_stride)
     if (width <= 256) LAUNCH(4);
     else if (width <= 512) LAUNCH(8);
     else if (width <= 1024) LAUNCH(16);

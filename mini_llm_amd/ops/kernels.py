@@ -815,7 +815,8 @@ def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activa
 # -- layers that norm after the sum, norm their heads, gate their feed-forward, or keep a latent -----------------
 def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool = False, out_dtype=None, row_index=None, with_stream: bool = False):
     """h / sqrt(mean(h^2) + eps) * g over rows of h = alpha * x (+ addend), g = weight or, with ``one_plus``, 1 + weight.
-    x: float32 [rows, width]; addend: float32 or bfloat16 of the same shape; weight: float32 [width]. ``row_index`` (int32)
+    x: float32 [rows, width]; addend: float32 or bfloat16 of the same shape, or float32 [n, rows, width], the partial products
+    of a product cut along K (``linear_split``), whose sum is the addend; weight: float32 [width]. ``row_index`` (int32)
     picks the input row of each output row. Returns the rows in ``out_dtype``, or with ``with_stream`` (the rows in float32:
     what a residual stream goes on with, the rows in ``out_dtype``); ``out_dtype`` None: the float32 rows alone."""
     _device_tensor(x, "x", torch.float32, 2)
@@ -823,16 +824,22 @@ def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool 
     width = x.shape[1]
     _require(weight.shape[0] == width, "the gain vector does not match the row width")
     n = x.shape[0]
+    n_partials, partial_stride = 1, 0
     if addend is not None:
-        _device_tensor(addend, "addend", dim=2)
-        _require(addend.shape == x.shape and row_index is None, "the addend must have the rows' shape (and rows are not gathered then)")
+        _device_tensor(addend, "addend")
+        if addend.dim() == 3:
+            _require(addend.dtype == torch.float32 and addend.shape[0] >= 1, "partial products are float32")
+            n_partials, partial_stride = addend.shape[0], addend.stride(0)
+        _require(tuple(addend.shape[-2:]) == tuple(x.shape) and addend.dim() in (2, 3) and row_index is None,
+                 "the addend must have the rows' shape (and rows are not gathered then)")
     if row_index is not None:
         _device_tensor(row_index, "row_index", torch.int32, 1)
         n = row_index.shape[0]
     stream = torch.empty((n, width), dtype=torch.float32, device=x.device) if with_stream or out_dtype is None else None
     rows = torch.empty((n, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
     check(library().mllm_rms_norm(_ptr(x), _ptr(addend), 0 if addend is None else _code(addend.dtype), float(alpha), _ptr(row_index), _ptr(weight),
-                                  int(bool(one_plus)), float(eps), _ptr(stream), _ptr(rows), 0 if rows is None else _code(rows.dtype), n, width, _stream()))
+                                  int(bool(one_plus)), float(eps), _ptr(stream), _ptr(rows), 0 if rows is None else _code(rows.dtype), n, width, n_partials,
+                                  partial_stride, _stream()))
     if out_dtype is None:
         return stream
     return (stream, rows) if with_stream else rows

@@ -13,7 +13,7 @@ import torch
 
 from ..ops import kernels
 from .base import KVNeed, LayerContext, Mixer, register_part
-from .linear import Linear
+from .linear import BranchProduct, Linear
 from .norms import LayerNorm
 
 
@@ -126,6 +126,7 @@ class NormedHeadAttention(Mixer):
         self.width, self.n_heads, self.n_kv_heads, self.dim, self.vdim = width, n_heads, n_kv_heads, dim, vdim
         self.scale, self.eps, self.temp_coef, self.temp_every, self.window, self.qk_norm = float(scale), float(eps), float(temp_coef), int(temp_every), window, qk_norm
         self.qkv = self.o = self.q_norm = self.k_norm = None
+        self._out_product = BranchProduct()
 
     def tensor_specs(self):
         from ..weights.spec import TABLE, VECTOR, Normal, TensorSpec
@@ -166,7 +167,7 @@ class NormedHeadAttention(Mixer):
             first_row=getattr(batch, "first_row", 0),
             **({"short_rows": batch.short_rows, "short_requests": batch.short_requests} if batch.short_portion <= kernels.DECODE_MAX_Q_LEN else {}),
         )
-        return kernels.linear(mixed, self.o, residual=residual, out_dtype=torch.float32)
+        return self._out_product(mixed, self.o, residual)
 
 
 register_part("mixer", "causal_attention", CausalSelfAttention)

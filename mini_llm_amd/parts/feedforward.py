@@ -8,7 +8,7 @@ import torch
 
 from ..ops import kernels
 from .base import FeedForward, register_part
-from .linear import Linear
+from .linear import BranchProduct, Linear
 from .norms import LayerNorm
 
 ACTIVATIONS = ("gelu_new", "gelu")
@@ -56,6 +56,7 @@ class GatedMLP(FeedForward):
         self.width, self.inner = width, inner
         self._names = names
         self.gate_up = self.down = None
+        self._down_product = BranchProduct()
 
     def tensor_specs(self):
         from ..weights.spec import MATRIX, TABLE, Normal, TensorSpec
@@ -72,7 +73,7 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, residual):
         inner = kernels.silu_mul(kernels.linear(x, self.gate_up))
-        return kernels.linear(inner, self.down, residual=residual, out_dtype=torch.float32)
+        return self._down_product(inner, self.down, residual)
 
 
 register_part("feed_forward", "dense_mlp", DenseMLP)

@@ -17,6 +17,7 @@ import torch
 from ..ops import kernels
 from ..weights.spec import TABLE, VECTOR, Normal, TensorSpec
 from .base import KVNeed, LayerContext, Mixer, register_part
+from .linear import BranchProduct
 from .positions import RotaryEncoding
 
 
@@ -33,6 +34,7 @@ class LatentAttention(Mixer):
         # a cached row: [latent | rotated key part | zeros up to a size the attention kernels take]
         self.row_size = kernels.latent_row_size(kv_rank + rot_dim)
         self.w_in = self.uk_t = self.uv = self.o = self.sink = self.dkv_norm = None
+        self._out_product = BranchProduct()
 
     def tensor_specs(self):
         H, std = self.n_heads, self.width ** -0.5
@@ -85,7 +87,7 @@ class LatentAttention(Mixer):
                                           context_lens=batch.context_lens, max_q_len=batch.max_q_len)
         mixed = torch.empty((rows, H, self.vdim), dtype=x.dtype, device=x.device)
         kernels.heads_linear(summed, self.uv, mixed, n_heads=H, k=self.kv_rank, x_head_stride=self.kv_rank, gate=gate)
-        return kernels.linear(mixed.view(rows, H * self.vdim), self.o, residual=residual, out_dtype=torch.float32)
+        return self._out_product(mixed.view(rows, H * self.vdim), self.o, residual)
 
 
 register_part("mixer", "latent_attention", LatentAttention)

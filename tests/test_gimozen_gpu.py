@@ -177,6 +177,23 @@ def test_generation_through_the_engine_and_its_scheduler(gimozen_dirs, dtype):
     np.testing.assert_allclose(first, want, atol=5e-5 if dtype == "float32" else 0.2, rtol=5e-5 if dtype == "float32" else 0.05)
 
 
+def test_the_command_line_completes_greedily(gimozen_dirs):
+    import subprocess
+    import sys
+
+    folder, config, weights = gimozen_dirs["attention"]
+    prompt = random_tokens(12, 9, config["vocab"])
+    done = subprocess.run([sys.executable, str(replay.ROOT / "bin" / "complete"), "--model", str(folder), "--dtype", "float32", "--temperature", "0",
+                           "--max-new-tokens", "12", "--max-length", "128", "--tokens", ",".join(map(str, prompt))], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    new = [int(t) for t in done.stdout.strip().split(",")]
+    logits = plain.forward(config, weights, prompt + new)
+    assert len(new) == 12
+    for k, token in enumerate(new):
+        row = logits[len(prompt) - 1 + k]
+        assert row[token] >= row.max() - 1e-4, (k, token, int(row.argmax()))
+
+
 def test_long_decoding_crosses_pages_and_key_runs(gimozen_dirs):
     # 700 decoded tokens, one by one, from captured steps: past ten pages and past the lengths at which the latent
     # attention cuts a row's keys into runs

@@ -45,6 +45,10 @@ def test_rms_norm_with_the_scaled_sum(width, one_plus):
     y16 = rounded(y, torch.bfloat16)
     got = k.rms_norm(gpu(x), gpu(w), 1e-5, addend=gpu(y, torch.bfloat16), alpha=1.5, one_plus=one_plus)
     np.testing.assert_allclose(got.cpu().numpy(), plain.rms_norm(1.5 * x + y16, w, 1e-5, one_plus), atol=2e-5, rtol=2e-5)
+    # the addend as the partial products of a product cut along K: the norm takes their sum
+    parts = rng.normal(0, 1, (3, 7, width))
+    got = k.rms_norm(gpu(x), gpu(w), 1e-5, addend=gpu(parts), alpha=1.5, one_plus=one_plus)
+    np.testing.assert_allclose(got.cpu().numpy(), plain.rms_norm(1.5 * x + parts.sum(axis=0), w, 1e-5, one_plus), atol=2e-5, rtol=2e-5)
     index = torch.tensor([6, 0, 3], dtype=torch.int32).cuda()
     got = k.rms_norm(gpu(x), gpu(w), 1e-5, one_plus=one_plus, out_dtype=torch.float32, row_index=index)
     np.testing.assert_allclose(got.cpu().numpy(), plain.rms_norm(x[[6, 0, 3]], w, 1e-5, one_plus), atol=2e-5, rtol=2e-5)
