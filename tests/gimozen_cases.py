@@ -36,4 +36,8 @@ CASES = {
     "latent": model([latent_layer(heads=1, dim=8, rot_dim=16, vdim=8, kv_rank=21, rot_dims=8, scaling=None),
                      latent_layer(heads=5, dim=24, rot_dim=4, vdim=16, kv_rank=64, base=500.0),
                      latent_layer(heads=2, dim=24, rot_dim=4, vdim=40, kv_rank=64, base=500.0, kv_from=1)], width=80, vocab=130, alpha=2.0),
+    # sizes that are no multiples of anything a kernel would like: rows of 200 bytes, heads of 20 and 12, a latent of 30 + 6
+    "odd": model([attention_layer(heads=5, kv_heads=1, dim=20, vdim=12, ff=90, every=3),
+                  latent_layer(heads=5, dim=20, rot_dim=6, vdim=12, kv_rank=30, ff=None, base=777.0),
+                  latent_layer(heads=7, dim=12, rot_dim=6, vdim=20, kv_rank=30, ff=90, base=777.0, kv_from=1)], width=100, vocab=77, alpha=0.7, eps=1e-6),
 }

@@ -46,7 +46,7 @@ def plain_logits(config, weights, requests, bf16):
     return {name: plain.forward(config, weights, tokens, stored=stored) for name, tokens in requests.items()}
 
 
-LENGTHS = {"mixed": [5, 130, 64, 65, 1, 200, 33], "attention": [2, 70, 129, 63, 40], "latent": [3, 300, 64, 17, 128, 66]}
+LENGTHS = {"mixed": [5, 130, 64, 65, 1, 200, 33], "attention": [2, 70, 129, 63, 40], "latent": [3, 300, 64, 17, 128, 66], "odd": [67, 2, 130, 31]}
 MODES = {"whole": replay.whole, "tail": replay.prefill_then_decode, "chunked": replay.chunked, "mixed": replay.mixed}
 # 32-bit: sums in another order than numpy's
 TOLERANCE = {"float32": dict(atol=5e-5, rtol=5e-5)}
