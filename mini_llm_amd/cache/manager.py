@@ -99,6 +99,15 @@ class CacheManager:
             pool.give([p for p in table if p != NO_PAGE])
         self._free_slots.append(entry.state_slot)
 
+    def snapshot_state(self) -> dict:
+        """A copy of every state layer as it stands (state layer -> tensor): for whoever has to run a step twice (once to warm
+        up before a capture, once for real) and must not move a recurrent state on twice."""
+        return {layer: tensor.clone() for layer, tensor in self.state.items()}
+
+    def restore_state(self, snapshot: dict) -> None:
+        for layer, tensor in snapshot.items():
+            self.state[layer].copy_(tensor)
+
     def length(self, request_id) -> int:
         return self._entry(request_id).length
 

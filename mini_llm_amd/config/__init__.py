@@ -1,6 +1,7 @@
 from .base import ConfigError, ModelConfig, read_config_json
 from .gimozen import GimozenConfig
 from .gpt2 import GPT2Config
+from .ketolix import KetolixConfig
 from .registry import (
     Architecture,
     architecture_name,
@@ -16,6 +17,7 @@ __all__ = [
     "ConfigError",
     "GimozenConfig",
     "GPT2Config",
+    "KetolixConfig",
     "ModelConfig",
     "architecture_name",
     "config_from_dict",

@@ -35,13 +35,29 @@ constexpr int MAX_HEAD = 256;
 // The general kernel: one wave per (token, head), any head size up to MAX_HEAD. Keys in tiles of
 // 64, a lane per key for the scores; softmax statistics in 32-bit, carried from tile to tile
 // (online softmax, as the reference's prefill kernel does: engine/src/attention.cu:71-124).
+// What a mixer may ask of the scores beyond scale, mask and softmax. softcap > 0: score <- softcap tanh(score / softcap),
+// behind the scale. sinks [n_heads]: exp(sink_h) joins the softmax's denominator of head h, once, with no key and no value.
+struct ScoreOptions {
+    float softcap;
+    const float* sinks;
+};
+
+// cap tanh(s / cap). EXACT: the library's tanhf; else 1 - 2 / (1 + e^(2x)) with the hardware's 2^x and reciprocal, for
+// scores that meet bfloat16 keys.
+template <bool EXACT>
+__device__ __forceinline__ float capped_score(float s, float cap) {
+    const float x = s / cap;
+    if constexpr (EXACT) return cap * tanhf(x);
+    return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * 2.8853900817779268f)));
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void attention_general_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int head_size, int page_size, int window, float scale) {
+    int head_size, int page_size, int window, float scale, ScoreOptions options) {
     __shared__ float q_shared[4][MAX_HEAD];
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
     const int token = blockIdx.x;
@@ -81,7 +97,7 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
             const T* k_row = k_pages + (size_t)row * head_size;
             float dot = 0.0f;
             for (int d = 0; d < head_size; d++) dot += my_q[d] * to_float(k_row[d]);
-            score = dot;
+            score = options.softcap > 0.0f ? capped_score<true>(dot, options.softcap) : dot;
         }
         float new_max = fmaxf(running_max, wave_max(score));
         float p = valid ? expf(score - new_max) : 0.0f;
@@ -102,6 +118,7 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
             }
         }
     }
+    if (options.sinks) running_sum += expf(options.sinks[head] - running_max);
     float inverse = 1.0f / running_sum;
 #pragma unroll
     for (int r = 0; r < REGS; r++) {
@@ -139,8 +156,9 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
                             void* out, int out_stride, const int* token_request,
                             const int* positions, const int* block_tables, int max_blocks,
                             int n_tokens, int n_heads, int n_kv_heads, int head_size, int page_size,
-                            int window, float scale, int dtype, hipStream_t stream) {
+                            int window, float scale, int dtype, float softcap, const float* sinks, hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention: bad sizes");
+    const ScoreOptions options = {softcap, sinks};
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention: %d heads do not divide into %d key/value heads",
                  n_heads, n_kv_heads);
     MLLM_REQUIRE(head_size > 0 && head_size <= MAX_HEAD,
@@ -155,12 +173,12 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
         attention_general_kernel<float><<<grid, 256, 0, stream>>>(
             (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, (float*)out,
             out_stride, token_request, positions, block_tables, max_blocks, n_heads, n_kv_heads,
-            head_size, page_size, window, scale);
+            head_size, page_size, window, scale, options);
     else if (dtype == MLLM_BF16)
         attention_general_kernel<bf16_t><<<grid, 256, 0, stream>>>(
             (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
             (bf16_t*)out, out_stride, token_request, positions, block_tables, max_blocks, n_heads,
-            n_kv_heads, head_size, page_size, window, scale);
+            n_kv_heads, head_size, page_size, window, scale, options);
     else
         MLLM_REQUIRE(false, "attention: unknown dtype %d", dtype);
     return mllm_check_launch("attention");
@@ -194,7 +212,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int page_shift, int window, float scale, int out_packed, float* parts_out, int* __restrict__ arrivals) {
+    int page_shift, int window, float scale, int out_packed, float* parts_out, int* __restrict__ arrivals, ScoreOptions options) {
     constexpr int VEC = KeySweep<T, HD>::VEC, LPR = KeySweep<T, HD>::LPR, RPI = KeySweep<T, HD>::RPI;
     __shared__ float partial[DECODE_MAX_SPLITS][HD + 2];
     __shared__ int through_last;
@@ -234,6 +252,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
 
     KeySweep<T, HD> sweep;
     sweep.init();
+    sweep.cap = options.softcap;
     if (begin < end && !TOGETHER) {
         // the plain order: the query, then round by round the pages, their rows, the softmax
         float qf[VEC];
@@ -317,7 +336,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
         const float run_sum = lane < n_parts ? far(lane * (HD + 2) + HD + 1) : 0.0f;
         const float all_max = wave_max_total(run_max);               // finite: the first run always has a key
         const float factor = run_max == -INFINITY ? 0.0f : expf(run_max - all_max);
-        const float one_over = 1.0f / wave_total(run_sum * factor);
+        const float one_over = 1.0f / (wave_total(run_sum * factor) + (options.sinks ? expf(options.sinks[head] - all_max) : 0.0f));
         for (int d0 = 0; d0 < HD; d0 += WAVE) {
             const int d = min(d0 + lane, HD - 1);
             float value = 0.0f;
@@ -332,6 +351,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
         }
         return;
     }
+    if (options.sinks) total += expf(options.sinks[head] - total_max);
     float inverse = 1.0f / total;
     for (int d = threadIdx.x; d < HD; d += blockDim.x) {
         float value = 0.0f;
@@ -345,7 +365,7 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
                     void* out, int out_stride, const int* token_request, const int* positions,
                     const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
                     int page_shift, int window, float scale, int n_splits, int out_packed, int n_parts, float* parts,
-                    int* arrivals, hipStream_t stream) {
+                    int* arrivals, ScoreOptions options, hipStream_t stream) {
     dim3 grid(n_heads, n_tokens, n_parts), block(WAVE * n_splits);
     // Measured on MI355X: starting with query and pages together (and, in bfloat16, the pages a
     // round ahead) is 3 to 15 % faster wherever a wave has few rounds, which is where a kernel's
@@ -362,11 +382,11 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
         if (together)                                                                                          \
             attention_decode_kernel<T, HD, true><<<grid, block, 0, stream>>>(                                  \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts, arrivals);  \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts, arrivals, options);  \
         else                                                                                                   \
             attention_decode_kernel<T, HD, false><<<grid, block, 0, stream>>>(                                 \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts, arrivals);  \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts, arrivals, options);  \
         return 0;
     switch (head_size) {
         MLLM_DECODE_CASE(16)
@@ -393,7 +413,8 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                                    const int* block_tables, int max_blocks, int n_tokens, int n_heads,
                                    int n_kv_heads, int head_size, int page_size, int window, float scale,
                                    int n_splits, int dtype, int out_packed, int n_parts, float* parts, int* arrivals,
-                                   hipStream_t stream) {
+                                   float softcap, const float* sinks, hipStream_t stream) {
+    const ScoreOptions options = {softcap, sinks};
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
@@ -412,10 +433,10 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
     int refused = 1;
     if (dtype == MLLM_F32)
         refused = dispatch_decode<float>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, arrivals, stream);
+                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, arrivals, options, stream);
     else
         refused = dispatch_decode<bf16_t>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, arrivals, stream);
+                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, arrivals, options, stream);
     MLLM_REQUIRE(!refused, "attention_decode: no kernel for dtype %d and head size %d", dtype, head_size);
     return mllm_check_launch("attention_decode");
 }
@@ -468,7 +489,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ q_starts, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int head_size, int page_shift, int window, float scale) {
+    int head_size, int page_shift, int window, float scale, ScoreOptions options) {
     typedef PrefillLds<T, HD_PAD, QG, KS> L;
     constexpr bool HALF = L::HALF;
     constexpr int VEC = HALF ? 8 : 4;
@@ -638,7 +659,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    s_acc[j][v] *= score_scale;
+                    s_acc[j][v] = options.softcap > 0.0f ? capped_score<!HALF>(s_acc[j][v] * scale, options.softcap) * (HALF ? LOG2E : 1.0f) : s_acc[j][v] * score_scale;
                     tile_max = fmaxf(tile_max, s_acc[j][v]);
                 }
         } else {
@@ -649,7 +670,8 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
                 for (int v = 0; v < 16; v++) {
                     int key = k0 + j * 32 + 8 * (v / 4) + 4 * half + (v % 4);
                     bool allowed = q_valid && key <= q_position && key >= first_allowed;
-                    float s = allowed ? s_acc[j][v] * score_scale : -INFINITY;
+                    float s = options.softcap > 0.0f ? capped_score<!HALF>(s_acc[j][v] * scale, options.softcap) * (HALF ? LOG2E : 1.0f) : s_acc[j][v] * score_scale;
+                    s = allowed ? s : -INFINITY;
                     s_acc[j][v] = s;
                     tile_max = fmaxf(tile_max, s);
                 }
@@ -741,9 +763,11 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc_o[i][v] += other[i * 16 + v] * w;
         }
+        running_max = safe_max;   // what the sums now stand at
     }
 
     if (!q_valid) return;
+    if (options.sinks) running_sum += softmax_exp<HALF>(options.sinks[head] * (HALF ? LOG2E : 1.0f) - running_max);
     float inverse = 1.0f / running_sum;  // every query sees at least its own key
     T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * head_size;
 #pragma unroll
@@ -759,7 +783,7 @@ template <typename T, int HD_PAD>
 void launch_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride,
                     const int* q_starts, const int* context_lens, const int* block_tables, int max_blocks,
                     int n_requests, int max_q_len, int n_heads, int n_kv_heads, int head_size, int page_shift,
-                    int window, float scale, hipStream_t stream) {
+                    int window, float scale, ScoreOptions options, hipStream_t stream) {
     // Queries per block (32*QG) set how often keys and values are read again from the cache;
     // waves along the keys (KS) set the length of the chain of dependent softmax updates.
     constexpr bool ROOMY = PrefillLds<T, HD_PAD, 1, 4>::TILE_BYTES <= 80 * 1024;
@@ -772,7 +796,7 @@ void launch_prefill(const void* q, int q_stride, const void* k_pages, const void
         mllm_count_kernel(MLLM_K_ATTENTION_PREFILL);                                                                   \
         attention_prefill_kernel<T, HD_PAD, QG, KS><<<grid, 64 * QG * KS, 0, stream>>>(                                \
             (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens, \
-            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_shift, window, scale);                      \
+            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_shift, window, scale, options);             \
     }
     if constexpr (ROOMY) {
         if (shape == 1) MLLM_PREFILL_LAUNCH(1, 4)
@@ -802,7 +826,9 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
                                     int out_stride, const int* q_starts, const int* context_lens,
                                     const int* block_tables, int max_blocks, int n_requests, int max_q_len,
                                     int max_len, int n_heads, int n_kv_heads, int head_size, int page_size, int window,
-                                    float scale, int dtype, hipStream_t stream) {
+                                    float scale, int dtype, float softcap, const float* sinks, hipStream_t stream) {
+    const ScoreOptions options = {softcap, sinks};
+    const bool plain_scores = softcap <= 0.0f && sinks == nullptr;   // the streaming kernels know scale, mask and softmax only
     // max_len: the longest sequence after this step, or a bound on it (0 or less: what the block tables can hold); it only
     // decides how many waves share a block's keys
     MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -818,20 +844,20 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
     while ((1 << page_shift) < page_size) page_shift++;
 #define MLLM_PREFILL_CASE(T, PAD)                                                                                      \
     launch_prefill<T, PAD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,      \
-                           max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_shift, window, scale, stream)
+                           max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_shift, window, scale, options, stream)
     const long table_reach = (long)max_blocks * page_size;
     const int reach = (int)(max_len > 0 && max_len < table_reach ? max_len : (table_reach < (1 << 30) ? table_reach : (1 << 30)));
 #define MLLM_STREAM_CASE(T, HD)                                                                                            \
     prefill_stream::launch<T, HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
                                   max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, stream)
-    if (dtype == MLLM_BF16 && prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+    if (plain_scores && dtype == MLLM_BF16 && prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
         // long portions, rows of 64 / 128 / 256 bytes, pages of 32 keys or more: keys and values stream from the pages straight into LDS
         if (head_size == 32) MLLM_STREAM_CASE(bf16_t, 32);
         else if (head_size == 64) MLLM_STREAM_CASE(bf16_t, 64);
         else MLLM_STREAM_CASE(bf16_t, 128);
         return mllm_check_launch("attention_prefill");
     }
-    if (dtype == MLLM_F32 && prefill_stream::takes<float>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+    if (plain_scores && dtype == MLLM_F32 && prefill_stream::takes<float>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
         if (head_size == 32) MLLM_STREAM_CASE(float, 32);
         else MLLM_STREAM_CASE(float, 64);
         return mllm_check_launch("attention_prefill");

@@ -47,12 +47,14 @@ struct KeySweep {
     float o[VEC];         // this lane's share of sum p * v, dimensions sub * VEC ..
     float running_max;    // the same in every lane
     float running_sum;    // this lane's share until merge_groups()
+    float cap;            // > 0: a score s counts as cap tanh(s / cap) (a caller that wants it sets it behind init())
 
     __device__ __forceinline__ void init() {
 #pragma unroll
         for (int i = 0; i < VEC; i++) o[i] = 0.0f;
         running_max = -INFINITY;
         running_sum = 0.0f;
+        cap = 0.0f;
     }
 
     // KPI keys as loaded: converted where they are used.
@@ -147,6 +149,10 @@ struct KeySweep {
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
             float dot = lanes_sum<LPR>(dots[u]);
+            if (cap > 0.0f) {
+                if constexpr (sizeof(T) == 2) dot = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(dot / cap * 2.8853900817779268f)));
+                else dot = cap * tanhf(dot / cap);
+            }
             score[u] = base + u * RPI + group < end ? dot : -INFINITY;
             tile_max = fmaxf(tile_max, score[u]);
         }

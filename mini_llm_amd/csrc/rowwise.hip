@@ -19,12 +19,15 @@ __device__ __forceinline__ void store_from_float(void* base, size_t index, int c
 // A wave per output row; a row
 // of up to 64 * REGS elements stays in registers between the two passes, a longer one is read again. row_index, if
 // given, names the input row of each output row. The result goes to `stream` (32-bit, what the residual stream goes on
-// with) and / or `rows` (the element type the next product reads); either may be null.
+// with) and / or `rows` (the element type the next product reads); either may be null. `residual` (32-bit, the output's
+// shape), if given, is added to the normed rows: out = residual + norm(h) g, the sum of a layer whose norm sits on its
+// branch's output.
 template <int REGS>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const void* __restrict__ y, int y_code, float alpha,
                                                        const int* __restrict__ row_index, const float* __restrict__ weight, int one_plus,
                                                        float eps, float* __restrict__ stream, void* __restrict__ rows, int rows_code,
-                                                       int n_rows, int width, int n_partials, long long partial_stride) {
+                                                       int n_rows, int width, int n_partials, long long partial_stride,
+                                                       const float* __restrict__ residual) {
     const int lane = threadIdx.x % WAVE;
     const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (row >= n_rows) return;
@@ -33,12 +36,13 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
     const float plus = one_plus ? 1.0f : 0.0f;
     if constexpr (REGS > 0) {
         // everything is asked for at once, from clamped places, so that the wave waits for memory once
-        float kept[REGS], added[REGS], gains[REGS];
+        float kept[REGS], added[REGS], gains[REGS], base[REGS];
 #pragma unroll
         for (int r = 0; r < REGS; r++) {
             const int i = min(lane + r * WAVE, width - 1);
             kept[r] = x[in_at + i];
             gains[r] = weight[i];
+            base[r] = residual ? residual[out_at + i] : 0.0f;
         }
         if (y) {
             if (y_code == MLLM_F32) {
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
         for (int r = 0; r < REGS; r++) {
             const int i = lane + r * WAVE;
             if (i < width) {
-                const float value = kept[r] * inverse * (plus + gains[r]);
+                const float value = base[r] + kept[r] * inverse * (plus + gains[r]);
                 if (stream) stream[out_at + i] = value;
                 if (rows) store_from_float(rows, out_at + i, rows_code, value);
             }
@@ -94,7 +98,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
         for (int i = lane; i < width; i += WAVE) {
             float h = alpha * x[in_at + i];
             for (int p = 0; y && p < n_partials; p++) h += load_as_float(y, p * partial_stride + in_at + i, y_code);
-            const float value = h * inverse * (plus + weight[i]);
+            const float value = (residual ? residual[out_at + i] : 0.0f) + h * inverse * (plus + weight[i]);
             if (stream) stream[out_at + i] = value;
             if (rows) store_from_float(rows, out_at + i, rows_code, value);
         }
@@ -307,7 +311,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ bot
 
 MLLM_API int mllm_rms_norm(const float* x, const void* y, int y_dtype, float alpha, const int* row_index, const float* weight, int one_plus,
                            float eps, float* stream_out, void* rows_out, int rows_dtype, int n_rows, int width, int n_partials,
-                           long long partial_stride, hipStream_t stream) {
+                           long long partial_stride, const float* residual, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && width > 0, "rms_norm: bad sizes rows=%d width=%d", n_rows, width);
     MLLM_REQUIRE(x != nullptr && weight != nullptr && (stream_out != nullptr || rows_out != nullptr), "rms_norm: a missing operand");
     MLLM_REQUIRE(y == nullptr || y_dtype == MLLM_F32 || y_dtype == MLLM_BF16, "rms_norm: unknown element type of the addend");
@@ -318,7 +322,7 @@ MLLM_API int mllm_rms_norm(const float* x, const void* y, int y_dtype, float alp
     if (n_rows == 0) return 0;
     const int waves = 4, blocks = ceil_div(n_rows, waves);
     mllm_count_kernel(MLLM_K_RMS_NORM);
-#define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width, n_partials, partial_stride)
+#define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width, n_partials, partial_stride, residual)
     if (width <= 256) LAUNCH(4);
     else if (width <= 512) LAUNCH(8);
     else if (width <= 1024) LAUNCH(16);

@@ -71,6 +71,7 @@ class StepBatch:
     groups: list            # GroupStepData per cache group
     request_ids: list = field(default_factory=list)
     host: dict = field(default_factory=dict)   # the same arrays as numpy, for parts that plan on the host
+    carry: dict = field(default_factory=dict)  # what a layer call leaves for a later call of the same step (rows of this batch)
 
     def rows_of_requests(self, lo: int, hi: int) -> "StepBatch":
         """Requests lo..hi-1 of a batch in which every request brings one token (a decode step) as a batch of their own,

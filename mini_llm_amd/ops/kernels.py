@@ -397,8 +397,10 @@ def _arrivals(k_pages, rows: int, n_heads: int):
 
 
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
-                    short_rows=None, short_requests=None, packed_out=False, first_row=0):
+                    short_rows=None, short_requests=None, packed_out=False, first_row=0, softcap: float = 0.0, sinks=None):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
+    ``softcap`` > 0: a scaled score s counts as softcap * tanh(s / softcap). ``sinks`` (float32 [n_heads]): exp(sink_h) joins
+    the denominator of head h's softmax, once, with no key and no value.
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
     row of block_tables that holds the request's pages (negative: padding row, output zero).
@@ -433,13 +435,18 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     lib = library()
     if n == 0:
         return out
+    if sinks is not None:
+        _device_tensor(sinks, "sinks", torch.float32, 1)
+        _require(sinks.shape[0] == n_heads, "one sink a head")
+    softcap = float(softcap or 0.0)
     rows_aligned = q.data_ptr() % 16 == 0 and (q.stride(0) * q.element_size()) % 16 == 0  # 16-byte loads of q
     if (short_rows is not None and short_requests is not None and 0 < short_rows < n and max_q_len is not None
             and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None and rows_aligned
             and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))
             and lib.mllm_attention_prefill_supported(head_size, page_size)):
         _require(0 < short_requests < context_lens.shape[0], "short_requests does not cut the batch in two")
-        common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len, first_row=first_row)
+        common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len, first_row=first_row,
+                      softcap=softcap, sinks=sinks)
         paged_attention(q[:short_rows], k_pages, v_pages, token_request, positions, block_tables, max_q_len=DECODE_MAX_Q_LEN,
                         q_starts=q_starts[: short_requests + 1], context_lens=context_lens[:short_requests],
                         out=out[:short_rows], **common)
@@ -476,7 +483,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), width if packed_out else out.stride(0),
                                         _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads,
                                         head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out),
-                                        n_parts, _ptr(parts), _ptr(arrivals), _stream()))
+                                        n_parts, _ptr(parts), _ptr(arrivals), softcap, _ptr(sinks), _stream()))
         return result
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):
@@ -485,9 +492,9 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         n_requests = context_lens.shape[0]
         _require(q_starts.shape[0] == n_requests + 1, "q_starts must have one entry more than context_lens")
         _require(block_tables.shape[0] >= n_requests, "fewer block tables than requests")
-        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
+        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), _stream()))
         return out
-    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
+    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), _stream()))
     return out
 
 
@@ -813,11 +820,13 @@ def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activa
 
 
 # -- layers that norm after the sum, norm their heads, gate their feed-forward, or keep a latent -----------------
-def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool = False, out_dtype=None, row_index=None, with_stream: bool = False):
+def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool = False, out_dtype=None, row_index=None, with_stream: bool = False,
+             residual=None):
     """h / sqrt(mean(h^2) + eps) * g over rows of h = alpha * x (+ addend), g = weight or, with ``one_plus``, 1 + weight.
     x: float32 [rows, width]; addend: float32 or bfloat16 of the same shape, or float32 [n, rows, width], the partial products
     of a product cut along K (``linear_split``), whose sum is the addend; weight: float32 [width]. ``row_index`` (int32)
-    picks the input row of each output row. Returns the rows in ``out_dtype``, or with ``with_stream`` (the rows in float32:
+    picks the input row of each output row. ``residual`` (float32, the output's shape) is added to the normed rows: residual +
+    norm(h) * g, the sum of a layer whose norm sits on its branch's output. Returns the rows in ``out_dtype``, or with ``with_stream`` (the rows in float32:
     what a residual stream goes on with, the rows in ``out_dtype``); ``out_dtype`` None: the float32 rows alone."""
     _device_tensor(x, "x", torch.float32, 2)
     _device_tensor(weight, "weight", torch.float32, 1)
@@ -835,11 +844,14 @@ def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool 
     if row_index is not None:
         _device_tensor(row_index, "row_index", torch.int32, 1)
         n = row_index.shape[0]
+    if residual is not None:
+        _device_tensor(residual, "residual", torch.float32, 2)
+        _require(tuple(residual.shape) == (n, width), "the residual must have the output's shape")
     stream = torch.empty((n, width), dtype=torch.float32, device=x.device) if with_stream or out_dtype is None else None
     rows = torch.empty((n, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
     check(library().mllm_rms_norm(_ptr(x), _ptr(addend), 0 if addend is None else _code(addend.dtype), float(alpha), _ptr(row_index), _ptr(weight),
                                   int(bool(one_plus)), float(eps), _ptr(stream), _ptr(rows), 0 if rows is None else _code(rows.dtype), n, width, n_partials,
-                                  partial_stride, _stream()))
+                                  partial_stride, _ptr(residual), _stream()))
     if out_dtype is None:
         return stream
     return (stream, rows) if with_stream else rows
@@ -997,4 +1009,139 @@ def latent_attention(q_full, pages, sinks, token_request, positions, block_table
     check(library().mllm_latent_attention(_ptr(q_full), _ptr(pages), _ptr(sinks), _ptr(out), _ptr(parts), _ptr(token_request), _ptr(positions),
                                           _ptr(block_tables), block_tables.shape[1], n, n_heads, int(rank), row_size, page_size, float(scale),
                                           n_runs, run_length, _code(pages.dtype), _stream()))
+    return out
+
+
+# -- mixers that norm whole projections, rotate neighbouring pairs, convolve over time or keep a matrix per head ------------
+def _rows_f32(t, name, width):
+    _require(isinstance(t, torch.Tensor) and t.is_cuda and t.dim() == 2 and t.dtype == torch.float32 and t.stride(1) == 1 and t.shape[1] == width,
+             f"{name} must be float32 GPU rows of {width} contiguous columns")
+
+
+def projection_rows(q, k, v, q_gain, k_gain, eps, frequencies, rot_dims, positions, slots, k_pages, v_pages, n_heads, n_kv_heads, dim, vdim, *,
+                    v_other=None, mix=None, write_cache: bool = True):
+    """The row-wise work between a mixer's projections and its attention. q [rows, n_heads * dim], k [rows, n_kv_heads * dim], v
+    [rows, n_kv_heads * vdim]: float32 views whose rows may be strided (parts of a fused product). Queries and keys are RMS-normed
+    over the whole projection with gain vectors of that length (None: no norm), then the first ``rot_dims`` elements of every head
+    rotated, element 2i with 2i + 1, by position * frequencies[i]. Returns q as [rows, n_heads * head_size] in the pages' type; keys
+    and values go to slots[row] of the pages ([num_pages, n_kv_heads, page_size, head_size], zeros beyond dim / vdim), the values
+    blended first where ``v_other`` (rows like v) and ``mix`` (a float32 number on the device) are given: (1 - mix) v + mix v_other."""
+    num_pages, n_kv, page_size, head_size = k_pages.shape
+    _check_pages(k_pages, v_pages, n_kv_heads, head_size)
+    n = q.shape[0]
+    _rows_f32(q, "q", n_heads * dim)
+    _rows_f32(k, "k", n_kv_heads * dim)
+    _rows_f32(v, "v", n_kv_heads * vdim)
+    _require(k.shape[0] == n and v.shape[0] == n, "q, k and v differ in rows")
+    _require(head_size >= dim and head_size >= vdim, "the pages' heads are too small")
+    for gain, name, width in ((q_gain, "q_gain", n_heads * dim), (k_gain, "k_gain", n_kv_heads * dim)):
+        if gain is not None:
+            _device_tensor(gain, name, torch.float32, 1)
+            _require(gain.shape[0] == width, f"{name} does not match the projection")
+    if rot_dims:
+        _device_tensor(frequencies, "frequencies", torch.float32, 1)
+        _require(rot_dims % 2 == 0 and rot_dims <= dim and frequencies.shape[0] >= rot_dims // 2, "the rotation does not fit the heads")
+    if v_other is not None:
+        _rows_f32(v_other, "v_other", n_kv_heads * vdim)
+        _device_tensor(mix, "mix", torch.float32)
+        _require(v_other.shape[0] == n and mix.numel() == 1, "the other values do not match")
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _device_tensor(slots, "slots", torch.int32, 1)
+    _require(positions.shape[0] >= n and slots.shape[0] >= n, "fewer positions or slots than rows")
+    out = torch.empty((n, n_heads * head_size), dtype=k_pages.dtype, device=q.device)
+    check(library().mllm_projection_rows(_ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(v_other), 0 if v_other is None else v_other.stride(0),
+                                         _ptr(mix if v_other is not None else None), _ptr(q_gain), _ptr(k_gain), float(eps), _ptr(frequencies if rot_dims else None),
+                                         int(rot_dims), _ptr(positions), _ptr(slots), _ptr(out), _ptr(k_pages), _ptr(v_pages), n, n_heads, n_kv_heads, dim, vdim,
+                                         head_size, page_size, int(bool(write_cache)), _code(k_pages.dtype), _stream()))
+    return out
+
+
+def head_gate(x, gate, out, n_heads, head_size, scale: float = 1.0):
+    """out[row, h, :] = x[row, h, :] * sigmoid(gate[row, h]) * scale. x, out: [rows, >= n_heads * head_size] of one element type (rows
+    may be strided); gate: float32 [rows, n_heads] (strided)."""
+    _require(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and out.dtype == x.dtype,
+             "x and out must be 2-D GPU tensors of one type with contiguous columns")
+    _rows_f32(gate, "gate", n_heads)
+    n = x.shape[0]
+    _require(out.shape[0] == n and gate.shape[0] == n and x.shape[1] >= n_heads * head_size and out.shape[1] >= n_heads * head_size, "the rows do not match the heads")
+    check(library().mllm_head_gate(_ptr(x), x.stride(0), _ptr(gate), gate.stride(0), float(scale), _ptr(out), out.stride(0), n, n_heads, head_size, _code(x.dtype), _stream()))
+    return out
+
+
+def gated_norm(x, weight, gate, eps, out, group: int | None = None, scale: float = 1.0):
+    """out = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate) * scale, the mean taken over each group of ``group`` neighbouring
+    elements (None: the whole row). x: float32 [rows, width]; weight: float32 [width] or None; gate: float32 [rows, width] (strided) or
+    None; out: [rows, >= width] (strided), any element type."""
+    width = x.shape[1]
+    _rows_f32(x, "x", width)
+    group = width if group is None else int(group)
+    if weight is not None:
+        _device_tensor(weight, "weight", torch.float32, 1)
+        _require(weight.shape[0] == width, "the gain vector does not match the rows")
+    if gate is not None:
+        _rows_f32(gate, "gate", width)
+        _require(gate.shape[0] == x.shape[0], "the gate does not match the rows")
+    _require(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == x.shape[0] and out.shape[1] >= width, "out does not match the rows")
+    check(library().mllm_gated_norm(_ptr(x), x.stride(0), _ptr(weight), _ptr(gate), 0 if gate is None else gate.stride(0), float(eps), float(scale), _ptr(out),
+                                    out.stride(0), x.shape[0], width, group, _code(out.dtype), _stream()))
+    return out
+
+
+def short_conv(u, weight, kept, token_request, q_starts, state_slots, keep: bool = True):
+    """A causal convolution over time on every channel: y_t = sum_j weight[c, j] * u_(t - taps + 1 + j). u: float32 [rows, channels]
+    (strided); weight: float32 [channels, taps]; ``kept``: float32 [slots, (taps - 1) * channels] (rows may be strided), each request's
+    last taps - 1 inputs in the order of time, read for the inputs before a portion's first row and, with ``keep``, moved on to the
+    sequence's new end. Returns y, float32 [rows, channels]."""
+    channels, taps = weight.shape
+    _device_tensor(weight, "weight", torch.float32, 2)
+    _rows_f32(u, "u", channels)
+    n = u.shape[0]
+    if taps > 1:
+        _rows_f32(kept, "kept", (taps - 1) * channels)
+    for t, name in ((token_request, "token_request"), (q_starts, "q_starts"), (state_slots, "state_slots")):
+        _device_tensor(t, name, torch.int32, 1)
+    n_requests = state_slots.shape[0]
+    _require(token_request.shape[0] >= n and q_starts.shape[0] >= n_requests + 1, "the batch's arrays are too short")
+    y = torch.empty((n, channels), dtype=torch.float32, device=u.device)
+    check(library().mllm_short_conv(_ptr(u), u.stride(0), _ptr(weight), taps, _ptr(kept) if taps > 1 else None, kept.stride(0) if taps > 1 else 0,
+                                    _ptr(token_request), _ptr(q_starts), _ptr(state_slots), _ptr(y), y.stride(0), n, n_requests, channels, int(bool(keep)), _stream()))
+    return y
+
+
+def recurrence_supported(dim: int, vdim: int) -> bool:
+    return bool(library().mllm_recurrence_supported(int(dim), int(vdim)))
+
+
+def recurrence(q, k, v, state, q_starts, state_slots, n_heads, dim, vdim, *, gate_in=None, gate_forget=None, cap: float = 0.0, decay=None,
+               q_scale: float = 1.0):
+    """A matrix per head and request, moved on row by row: S <- a S + b k v^T, o = S^T q, all in 32-bit. q, k: float32 [rows, n_heads *
+    dim]; v: [rows, n_heads * vdim] (strided views); ``state``: float32 [slots, >= what the kind keeps] (rows may be strided);
+    the rows of request r are q_starts[r] .. q_starts[r + 1], its state in slot state_slots[r] (negative: skipped).
+    With ``gate_in`` / ``gate_forget`` (float32 [rows, n_heads], the sums of the gates' projections): the matrix memory of an mLSTM, the
+    gates capped at +-cap (0: not), a normaliser and a running maximum kept behind the matrices ([heads, dim, vdim], [heads, dim],
+    [heads]). With ``decay`` (float32 [n_heads]): a = decay_h, b = 1, and q, k, v go through silu. Returns o, float32 [rows, n_heads * vdim]."""
+    _rows_f32(q, "q", n_heads * dim)
+    _rows_f32(k, "k", n_heads * dim)
+    _rows_f32(v, "v", n_heads * vdim)
+    n = q.shape[0]
+    _require(k.shape[0] == n and v.shape[0] == n, "q, k and v differ in rows")
+    _require(state.is_cuda and state.dim() == 2 and state.dtype == torch.float32 and state.stride(1) == 1, "the state must be float32 rows on the GPU")
+    _device_tensor(q_starts, "q_starts", torch.int32, 1)
+    _device_tensor(state_slots, "state_slots", torch.int32, 1)
+    n_requests = state_slots.shape[0]
+    _require(q_starts.shape[0] >= n_requests + 1, "q_starts must have one entry more than there are requests")
+    matrices = n_heads * dim * vdim
+    gated = gate_in is not None
+    if gated:
+        _rows_f32(gate_in, "gate_in", n_heads)
+        _rows_f32(gate_forget, "gate_forget", n_heads)
+        _require(gate_in.shape[0] == n and gate_forget.shape[0] == n and gate_in.stride(0) == gate_forget.stride(0), "the gates do not match the rows")
+        _require(state.shape[1] >= matrices + n_heads * dim + n_heads, "the state is too small for matrices, normalisers and maxima")
+    else:
+        _device_tensor(decay, "decay", torch.float32, 1)
+        _require(decay.shape[0] == n_heads and state.shape[1] >= matrices, "one decay a head, and a state that holds the matrices")
+    out = torch.empty((n, n_heads * vdim), dtype=torch.float32, device=q.device)
+    check(library().mllm_recurrence(0 if gated else 1, _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), _ptr(gate_forget),
+                                    gate_in.stride(0) if gated else 0, float(cap or 0.0), _ptr(decay), float(q_scale), _ptr(state), state.stride(0), matrices,
+                                    matrices + n_heads * dim, _ptr(q_starts), _ptr(state_slots), _ptr(out), out.stride(0), n_requests, n_heads, dim, vdim, _stream()))
     return out

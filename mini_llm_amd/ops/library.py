@@ -29,10 +29,10 @@ _SIGNATURES = {
     "mllm_probe_read": [P, c_longlong, P, c_int, P],
     "mllm_probe_mfma": [P, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
-    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, P, P, P],
+    "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_float, P, P],
+    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, P, P, c_float, P, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
-    "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_float, P, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P, P, P],
     "mllm_gemm_best_per_row": [c_int, c_int, c_int, c_int],
@@ -47,7 +47,7 @@ _SIGNATURES = {
     "mllm_linear_split_static": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_static_scratch_prepare": [],
     "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
-    "mllm_rms_norm": [P, P, c_int, c_float, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_longlong, P],
+    "mllm_rms_norm": [P, P, c_int, c_float, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_longlong, P, P],
     "mllm_head_norm": [P, c_int, P, P, c_float, c_float, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_latent_rows": [P, c_int, P, c_int, P, c_float, P, c_float, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_silu_mul": [P, P, c_int, c_int, c_int, P],
@@ -58,6 +58,14 @@ _SIGNATURES = {
     "mllm_latent_attention_mfma_supported": [c_int, c_int, c_int],
     "mllm_latent_attention_mfma": [P, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
     "mllm_latent_attention": [P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
+    "mllm_projection_rows": [P, c_int, P, c_int, P, c_int, P, c_int, P, P, P, c_float, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_int, c_int, P],
+    "mllm_head_gate": [P, c_int, P, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gated_norm": [P, c_int, P, P, c_int, c_float, c_float, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_short_conv": [P, c_int, P, c_int, P, c_longlong, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_recurrence_supported": [c_int, c_int],
+    "mllm_recurrence": [c_int, P, c_int, P, c_int, P, c_int, P, P, c_int, c_float, P, c_float, P, c_longlong, c_longlong, c_longlong, P, P, P, c_int, c_int,
+                        c_int, c_int, c_int, P],
 }
 
 

@@ -4,18 +4,21 @@ from .base import (
     Block, FeedForward, KVNeed, LayerContext, Mixer, Norm, Part, PositionEncoding, StateNeed,
     make_part, register_part,
 )
-from .block import PostNormBlock, PreNormBlock
+from .block import BranchNormBlock, PostNormBlock, PreNormBlock
 from .embedding import LinearHead, TiedHead, TokenEmbedding
 from .feedforward import DenseMLP, GatedMLP
 from .latent_attention import LatentAttention
 from .linear import Linear
 from .norms import LayerNorm, RMSNorm
 from .positions import LearnedPositions, RotaryEncoding
+from .projection_attention import ProjectionNormAttention
+from .recurrent import DecayedLinearAttention, MatrixMemoryMixer, ParallelMixer
 
 __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS",
     "Block", "FeedForward", "KVNeed", "LayerContext", "Mixer", "Norm", "Part", "PositionEncoding", "StateNeed",
     "make_part", "register_part",
     "CausalSelfAttention", "PreNormBlock", "TiedHead", "TokenEmbedding", "DenseMLP", "Linear", "LayerNorm", "LearnedPositions",
-    "NormedHeadAttention", "LatentAttention", "PostNormBlock", "LinearHead", "GatedMLP", "RMSNorm", "RotaryEncoding",
+    "NormedHeadAttention", "LatentAttention", "BranchNormBlock", "ProjectionNormAttention", "DecayedLinearAttention",
+    "MatrixMemoryMixer", "ParallelMixer", "PostNormBlock", "LinearHead", "GatedMLP", "RMSNorm", "RotaryEncoding",
 ]

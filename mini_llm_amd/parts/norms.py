@@ -61,6 +61,19 @@ class RMSNorm(Norm):
         return kernels.NormedRows(*kernels.rms_norm(x, self.weight, self.eps, addend=addend, alpha=alpha, one_plus=self.one_plus,
                                                     out_dtype=out_dtype, with_stream=True))
 
+    def forward_onto(self, stream, branch, out_dtype):
+        """stream + norm(branch) -> kernels.NormedRows: the sum of a layer whose norm sits on its branch's output, in float32 and in
+        ``out_dtype``, from one kernel. ``branch``: float32 rows, or the partial products [n, rows, width] of a product cut along K,
+        which are added up on the way in."""
+        addend = None
+        if branch.dim() == 3:
+            branch, addend = branch[0], (branch[1:] if branch.shape[0] > 1 else None)
+        if out_dtype == stream.dtype:
+            total = kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream)
+            return kernels.NormedRows(total, total)
+        return kernels.NormedRows(*kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream,
+                                                    out_dtype=out_dtype, with_stream=True))
+
 
 register_part("norm", "layernorm", LayerNorm)
 register_part("norm", "rmsnorm", RMSNorm)

@@ -22,29 +22,39 @@ class LearnedPositions(PositionEncoding):
 
 
 class RotaryEncoding(PositionEncoding):
-    """Rotation of the first ``dims`` elements of a head by an angle that grows with the position, element i paired with
-    element i + dims / 2 ("rotate half"): pair i turns by p * f_i with f_i = base^(-2i / dims). It has no tensors; the mixer
-    that holds it applies it to its queries and keys (``stage`` "mixer") with ``frequencies`` and ``magnitude``.
+    """Rotation of the first ``dims`` elements of a head by an angle that grows with the position: pair i turns by p * f_i with
+    f_i = base^(-2i / dims). ``pairing`` says which elements make pair i: "half" pairs element i with element i + dims / 2,
+    "neighbours" pairs element 2i with element 2i + 1, (u, v) -> (u cos a - v sin a, v cos a + u sin a). It has no tensors; the
+    mixer that holds it applies it to its queries and keys (``stage`` "mixer") with ``frequencies`` and ``magnitude``.
 
-    ``scaling`` = {factor, original, fast, slow} stretches the slow pairs for sequences longer than ``original`` positions
-    (YaRN: Peng, Quesnelle, Fan, Shippole, "YaRN: Efficient Context Window Extension of Large Language Models"): with
-    pair(t) = dims * ln(original / (2 pi t)) / (2 ln base), the pair that turns t times within the original length, lo =
-    max(floor(pair(fast)), 0), hi = min(ceil(pair(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
-    the frequency becomes f_i / factor * ramp_i + f_i * (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    ``scaling`` stretches the slow pairs for sequences longer than ``original`` positions, in one of two ways (``kind``):
+
+    "yarn" (the default), {factor, original, fast, slow} (YaRN: Peng, Quesnelle, Fan, Shippole, "YaRN: Efficient Context Window
+    Extension of Large Language Models"): with pair(t) = dims * ln(original / (2 pi t)) / (2 ln base), the pair that turns t
+    times within the original length, lo = max(floor(pair(fast)), 0), hi = min(ceil(pair(slow)), dims - 1) and ramp_i =
+    clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency becomes f_i / factor * ramp_i + f_i * (1 - ramp_i), and cos and
+    sin are multiplied by 0.1 ln(factor) + 1.
+
+    "wavelength", {factor, low, high, original}: by a pair's wavelength l = 2 pi / f. A pair with l < original / high keeps f; one
+    with l > original / low gets f / factor; between the two, with s = (original / l - low) / (high - low), the frequency is
+    (1 - s) f / factor + s f. cos and sin keep their size."""
 
     stage = "mixer"
 
-    def __init__(self, dims: int, base: float, scaling: dict | None = None):
+    def __init__(self, dims: int, base: float, scaling: dict | None = None, pairing: str = "half"):
         import math
 
         if dims < 0 or dims % 2:
             raise ValueError(f"a rotation pairs elements: {dims} is not an even number of them")
         if not base > 0:
             raise ValueError(f"the base must be positive, not {base}")
-        self.dims, self.base, self.scaling = dims, float(base), dict(scaling) if scaling else None
+        if pairing not in ("half", "neighbours"):
+            raise ValueError(f"unknown pairing {pairing!r}: half or neighbours")
+        self.dims, self.base, self.scaling, self.pairing = dims, float(base), dict(scaling) if scaling else None, pairing
         values = [self.base ** (-2.0 * i / dims) for i in range(dims // 2)]
         self.magnitude = 1.0
-        if self.scaling:
+        kind = (self.scaling or {}).get("kind", "yarn")
+        if self.scaling and kind == "yarn":
             factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
             pair = lambda turns: dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
             lo = max(math.floor(pair(float(self.scaling["fast"]))), 0)
@@ -53,6 +63,20 @@ class RotaryEncoding(PositionEncoding):
                 ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
                 values[i] = f / factor * ramp + f * (1.0 - ramp)
             self.magnitude = 0.1 * math.log(factor) + 1.0
+        elif self.scaling and kind == "wavelength":
+            factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+            low, high = float(self.scaling["low"]), float(self.scaling["high"])
+            for i, f in enumerate(values):
+                wavelength = 2.0 * math.pi / f
+                if wavelength < original / high:
+                    continue
+                if low > 0 and wavelength > original / low:   # (with low = 0 no wavelength is past original / low)
+                    values[i] = f / factor
+                else:
+                    s = (original / wavelength - low) / (high - low)
+                    values[i] = (1.0 - s) * f / factor + s * f
+        elif self.scaling:
+            raise ValueError(f"unknown kind of scaling {kind!r}: yarn or wavelength")
         self.values = values   # float64 on the host; ``frequencies`` rounds them to 32-bit on the device
         self._on_device = {}
 
