@@ -180,9 +180,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 // there yet: the host brings the table before that step runs), its token source becomes its own
 // slot, and its entry of draw_counts (if given: how many tokens the row's request has drawn, which the
 // sampler's random numbers are a function of) grows by one. A block takes 16 rows, a wave a row.
+constexpr int MAX_STEP_GROUPS = 16;   // cache groups a step may have to be moved on by the device
 struct StepGroups {
-    const int* tables[4];
-    int* slots[4];
+    const int* tables[MAX_STEP_GROUPS];
+    int* slots[MAX_STEP_GROUPS];
     int count, table_width, page_shift;
 };
 
@@ -307,7 +308,7 @@ MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, i
     StepGroups groups{};
     if (advance) {
         MLLM_REQUIRE(positions && context_lens && token_sources, "choose: nothing to advance");
-        MLLM_REQUIRE(n_groups >= 0 && n_groups <= 4, "choose: %d cache groups, at most 4 are advanced on the device", n_groups);
+        MLLM_REQUIRE(n_groups >= 0 && n_groups <= MAX_STEP_GROUPS, "choose: %d cache groups, at most %d are advanced on the device", n_groups, MAX_STEP_GROUPS);
         MLLM_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0 && (n_groups == 0 || table_width > 0), "choose: bad page size or table width");
         for (int g = 0; g < n_groups; g++) {
             MLLM_REQUIRE(group_tables[g] && group_slots[g], "choose: group %d has no table or slots", g);

@@ -615,7 +615,7 @@ def choose(values, indices, state_slots, token_slots, out=None, host_ring=None, 
             _device_tensor(t, name, torch.int32, 1)
             _require(t.shape[0] >= rows, f"{name} has fewer entries than rows")
         n_groups, page_size = len(advance.block_tables), int(advance.page_size)
-        _require(len(advance.slots) == n_groups and n_groups <= 4, "one row of slots per block table, at most four groups")
+        _require(len(advance.slots) == n_groups and n_groups <= 16, "one row of slots per block table, at most sixteen groups")
         import ctypes
 
         for g, (table, slot) in enumerate(zip(advance.block_tables, advance.slots)):

@@ -238,7 +238,7 @@ def read_safetensors(path) -> dict:
 def write_safetensors(path, tensors: dict, bf16: bool = False) -> None:
     header, chunks, offset = {}, [], 0
     for name, arr in tensors.items():
-        arr = np.ascontiguousarray(arr)
+        arr = np.ascontiguousarray(arr).reshape(np.shape(arr))   # (a number without dimensions stays one)
         if bf16 and arr.dtype == np.float32:
             data, dt = f32_to_bf16_rne(arr).tobytes(), "BF16"
         else:

@@ -51,7 +51,7 @@ def rotary_frequencies(rot: dict) -> np.ndarray:
             wavelength = 2.0 * np.pi / fi
             if wavelength < original / high:
                 out[i] = fi
-            elif wavelength > original / low:
+            elif low > 0 and wavelength > original / low:
                 out[i] = fi / factor
             else:
                 s = (original / wavelength - low) / (high - low)
@@ -235,3 +235,92 @@ def forward(config: dict, tensors: dict, tokens, round_to=None, layers_out: list
             layers_out.append(x.copy())
     x = rms_unit(x, eps) * tensors["final.norm"]
     return product(x, tensors["embed"], rnd)
+
+
+def greedy(config: dict, tensors: dict, prompt, n_new: int, round_to=None) -> list:
+    tokens = list(prompt)
+    for _ in range(n_new):
+        tokens.append(int(forward(config, tensors, tokens, round_to)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+# -- random models for the tests ------------------------------------------------------------------------------------------
+def tensor_shapes(config: dict) -> dict:
+    """name -> shape of every tensor a model of this configuration has."""
+    width = int(config["width"])
+    shapes = {"embed": (int(config["vocab"]), width), "final.norm": (width,)}
+    for index, layer in enumerate(config["layers"]):
+        p, m = f"l{index}.", layer["mixer"]
+        shapes[p + "norm1"] = (width,)
+        if layer["type"] == "mlstm":
+            H, d, e = m["heads"], m["dim"], m["vdim"]
+            shapes.update({p + "mix.q": (H * d, width), p + "mix.k": (H * d, width), p + "mix.v": (H * e, width), p + "mix.g": (H * e, width),
+                           p + "mix.o": (width, H * e), p + "mix.norm": (H * e,), p + "mix.i": (H, width), p + "mix.i.b": (H,),
+                           p + "mix.f": (H, width), p + "mix.f.b": (H,)})
+        elif layer["type"] == "attention":
+            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            shapes.update({p + "mix.q": (H * d, width), p + "mix.k": (G * d, width), p + "mix.v": (G * e, width), p + "mix.q.norm": (H * d,),
+                           p + "mix.k.norm": (G * d,), p + "mix.sink": (H,), p + "mix.o": (width, H * e)})
+            if m.get("v_mix"):
+                shapes[p + "mix.vmix"] = ()
+        elif layer["type"] == "parallel":
+            left, right = m["left"], m["right"]
+            H, G, d = left["heads"], left["kv_heads"], left["dim"]
+            shapes.update({p + "mix.left.q": (H * d, width), p + "mix.left.q.b": (H * d,), p + "mix.left.k": (G * d, width), p + "mix.left.k.b": (G * d,),
+                           p + "mix.left.q.norm": (H * d,), p + "mix.left.k.norm": (G * d,), p + "mix.left.g": (H, width),
+                           p + "mix.left.o": (width, H * d), p + "mix.left.o.b": (width,)})
+            if left.get("conv"):
+                shapes.update({p + "mix.left.q.conv": (H * d, left["conv"]), p + "mix.left.k.conv": (G * d, left["conv"])})
+            H, d, e = right["heads"], right["dim"], right["vdim"]
+            shapes.update({p + "mix.right.q": (H * d, width), p + "mix.right.k": (H * d, width), p + "mix.right.v": (H * e, width),
+                           p + "mix.right.g": (H * e, width), p + "mix.right.o": (width, H * e), p + "mix.right.norm": (H * e,)})
+        if layer.get("mlp"):
+            ff = layer["mlp"]["ff"]
+            shapes.update({p + "norm2": (width,), p + "mlp.gate": (ff, width), p + "mlp.up": (ff, width), p + "mlp.down": (width, ff)})
+    return shapes
+
+
+def random_weights(config: dict, seed: int) -> dict:
+    """Weights whose activations stay of order one: matrices ~ N(0, 1/in), gains around one, biases and sinks of order one, forget
+    biases well above zero. float32 arrays holding bfloat16 values (as files hold them)."""
+    import plain_gpt2
+
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(config).items():
+        last = name.rsplit(".", 1)[-1]
+        if name.endswith(".sink"):
+            value = rng.normal(0.0, 1.0, shape)
+        elif name.endswith(".vmix"):
+            value = rng.uniform(0.2, 0.8, shape)
+        elif name.endswith(".f.b"):
+            value = rng.normal(3.0, 0.5, shape)
+        elif name.endswith(".conv"):
+            value = rng.normal(0.0, shape[1] ** -0.5, shape)
+        elif last in ("norm", "norm1", "norm2"):
+            value = 1.0 + rng.normal(0.0, 0.1, shape)
+        elif last == "b":
+            value = rng.normal(0.0, 0.3, shape)
+        elif name == "embed":
+            value = rng.normal(0.0, 1.0, shape)
+        else:
+            value = rng.normal(0.0, shape[1] ** -0.5, shape)
+        out[name] = plain_gpt2.round_to_bf16(np.asarray(value, dtype=np.float32))
+    return out
+
+
+def as_float64(weights: dict) -> dict:
+    return {name: np.asarray(value, dtype=np.float64) for name, value in weights.items()}
+
+
+def write_model_dir(path, config: dict, weights: dict):
+    import json
+    from pathlib import Path
+
+    import plain_gpt2
+
+    path = Path(path)
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(config, indent=1))
+    plain_gpt2.write_safetensors(path / "model.safetensors", {k: np.asarray(v, dtype=np.float32) for k, v in weights.items()}, bf16=True)
+    return path
