@@ -339,7 +339,9 @@ DESIGN_SIZES = {   # width, layers; heads of 64; GPT-2's inner size 4 x width, t
 _KERNEL_CLASSES = {
     "products": ("gemm", "gemm_split", "gemm_qkv_cache", "gemm_best", "heads_linear"),
     "attention": ("attention", "attention_decode", "attention_prefill", "latent_attention"),
-    "row-wise": ("layernorm", "pending_layernorm", "rms_norm", "head_norm", "latent_rows", "silu_mul", "pending_sum", "add", "cache_write", "embed"),
+    "row-wise": ("layernorm", "pending_layernorm", "rms_norm", "head_norm", "latent_rows", "silu_mul", "pending_sum", "add", "cache_write", "embed",
+                 "projection_rows", "head_gate", "gated_norm", "short_conv"),
+    "recurrence": ("recurrence",),
     "layer kernels": ("decode_attention_half", "decode_mlp_half"),
     "choice": ("choose", "sample"),
 }
@@ -368,9 +370,31 @@ def gimozen_shape(width: int, layers: int, vocab: int = 50257) -> dict:
             "postln_alpha": 1.0, "layers": out}
 
 
+def ketolix_shape(width: int, layers: int, vocab: int = 50257) -> dict:
+    """Layers in fours: a matrix memory (heads of 64 x 128), two attention layers (heads of 64, a key/value head for every four,
+    a window of 512, a softcap, a sink, rotation with stretched wavelengths, values mixed with the first such layer's), and
+    attention beside a decayed recurrence (heads of 64 whose values are their keys, behind a convolution of four taps; heads of
+    64 x 128 with decays from 0.9 to 0.999); feed-forwards of 8/3 x width."""
+    heads, wide_heads = width // 64, max(1, width // 128)
+    ff = -(-(8 * width // 3) // 64) * 64
+    rot = {"dims": 64, "base": 50000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}}
+    mlp = {"kind": "dense", "ff": ff}
+    attention = {"type": "attention", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "softcap": 30.0,
+                                                           "mask": {"size": 512}, "rot": rot, "v_mix": True}}
+    memory = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": wide_heads, "dim": 64, "vdim": 128, "gate_cap": 15.0}}
+    decays = [1.0 - 0.1 ** (1.0 + 2.0 * i / max(1, wide_heads - 1)) for i in range(wide_heads)]
+    parallel = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "conv": 4, "mask": {"size": 512},
+                 "rot": {"dims": 32, "base": 50000.0}},
+        "right": {"heads": wide_heads, "dim": 64, "vdim": 128, "decay": decays}, "left_scale": 0.7, "right_scale": 0.7}}
+    pattern = [memory, attention, attention, parallel]
+    return {"architecture": "Ketolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": [pattern[i % 4] for i in range(layers)]}
+
+
 def measure_design(args) -> dict:
-    """Prefill and decode throughput of the Gimozen design and of GPT-2 with as many layers of the same width (random
-    weights), and where each model's step spends its time, by class of kernel, inside a prompt step and a decode step."""
+    """Prefill and decode throughput of a design and of the framework's closest older model with as many layers of the same width
+    (random weights): Gimozen beside GPT-2, Ketolix beside Gimozen; and where each model's step spends its time, by class of
+    kernel, inside a prompt step and a decode step."""
     import numpy as np
     import torch
 
@@ -379,10 +403,13 @@ def measure_design(args) -> dict:
     from mini_llm_amd.engine.engine import Engine, EngineOptions
 
     width, layers = DESIGN_SIZES[args.shape]
-    raws = {"gimozen": gimozen_shape(width, layers),
-            "gpt2": {"architectures": ["GPT2LMHeadModel"], "n_layer": layers, "n_embd": width, "n_head": width // 64, "n_inner": 4 * width,
-                     "vocab_size": 50257, "n_positions": CONTEXT, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}}
-    record = {"design": "gimozen beside gpt2", "width": width, "layers": layers, "dtype": args.dtype, "context": CONTEXT, "prompt_len": args.prompt_len}
+    if args.design == "ketolix":
+        raws = {"ketolix": ketolix_shape(width, layers), "gimozen": gimozen_shape(width, layers)}
+    else:
+        raws = {"gimozen": gimozen_shape(width, layers),
+                "gpt2": {"architectures": ["GPT2LMHeadModel"], "n_layer": layers, "n_embd": width, "n_head": width // 64, "n_inner": 4 * width,
+                         "vocab_size": 50257, "n_positions": CONTEXT, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}}
+    record = {"design": " beside ".join(raws), "width": width, "layers": layers, "dtype": args.dtype, "context": CONTEXT, "prompt_len": args.prompt_len}
     rng = np.random.default_rng(SEED + 7)
     for name, raw in raws.items():
         config = config_from_dict(raw)
@@ -641,8 +668,8 @@ def main() -> int:
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
     parser.add_argument("--step-by-step", action="store_true", help="--serving reads every step's tokens before it launches the next")
-    parser.add_argument("--design", default=None, choices=("gimozen",), help="the Gimozen design beside GPT-2 with as many layers of the same width (--shape small|medium): "
-                        "prefill and decode throughput of both, and where their steps spend the time")
+    parser.add_argument("--design", default=None, choices=("gimozen", "ketolix"), help="a design beside the closest older model with as many layers of the same width "
+                        "(--shape small|medium): Gimozen beside GPT-2, Ketolix beside Gimozen; prefill and decode throughput of both, and where their steps spend the time")
     parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:

@@ -235,11 +235,13 @@ def _capture(runner, batch, choice=None, lanes=None):
         warm["choice"] = replace(choice, token_slots=torch.empty_like(choice.token_slots), host_ring=None, cursor=None, advance=False)
     side = torch.cuda.Stream(device=runner.device)
     side.wait_stream(torch.cuda.current_stream())
-    kept_state = runner.cache.snapshot_state()   # a mixer that keeps state moves it on in place: the warm-up must not count
+    cache = getattr(runner, "cache", None)
+    kept_state = cache.snapshot_state() if cache is not None else None   # a mixer that keeps state moves it on in place: the warm-up must not count
     with torch.cuda.stream(side):
         runner.forward(batch, **warm)
     torch.cuda.current_stream().wait_stream(side)
-    runner.cache.restore_state(kept_state)
+    if kept_state:
+        cache.restore_state(kept_state)
     torch.cuda.synchronize(runner.device)
     graph = torch.cuda.CUDAGraph()
     # No garbage collection while the stream is being captured: it may finalise whatever lies around in reference

@@ -30,6 +30,13 @@ def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page_size=None, time
     out_dir = Path(out_dir)
     cmd = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
            "--out", str(out_dir), "--max-tokens", str(max_tokens)]
+    live, most = set(), 4   # state slots: as many as requests are live at once (the runner's own default is four)
+    for s in steps:
+        live |= {e["id"] for e in s["entries"]}
+        most = max(most, len(live))
+        live -= set(s["end"])
+    if most > 4:
+        cmd += ["--max-requests", str(most)]
     if page_size:
         cmd += ["--page-size", str(page_size)]
     if hidden_out:
