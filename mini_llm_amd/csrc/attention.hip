@@ -828,7 +828,6 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
                                     int max_len, int n_heads, int n_kv_heads, int head_size, int page_size, int window,
                                     float scale, int dtype, float softcap, const float* sinks, hipStream_t stream) {
     const ScoreOptions options = {softcap, sinks};
-    const bool plain_scores = softcap <= 0.0f && sinks == nullptr;   // the streaming kernels know scale, mask and softmax only
     // max_len: the longest sequence after this step, or a bound on it (0 or less: what the block tables can hold); it only
     // decides how many waves share a block's keys
     MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -849,15 +848,15 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
     const int reach = (int)(max_len > 0 && max_len < table_reach ? max_len : (table_reach < (1 << 30) ? table_reach : (1 << 30)));
 #define MLLM_STREAM_CASE(T, HD)                                                                                            \
     prefill_stream::launch<T, HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
-                                  max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, stream)
-    if (plain_scores && dtype == MLLM_BF16 && prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+                                  max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, options, stream)
+    if (dtype == MLLM_BF16 && prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
         // long portions, rows of 64 / 128 / 256 bytes, pages of 32 keys or more: keys and values stream from the pages straight into LDS
         if (head_size == 32) MLLM_STREAM_CASE(bf16_t, 32);
         else if (head_size == 64) MLLM_STREAM_CASE(bf16_t, 64);
         else MLLM_STREAM_CASE(bf16_t, 128);
         return mllm_check_launch("attention_prefill");
     }
-    if (plain_scores && dtype == MLLM_F32 && prefill_stream::takes<float>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+    if (dtype == MLLM_F32 && prefill_stream::takes<float>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
         if (head_size == 32) MLLM_STREAM_CASE(float, 32);
         else MLLM_STREAM_CASE(float, 64);
         return mllm_check_launch("attention_prefill");

@@ -164,7 +164,7 @@ template <typename T, int HD, int QUERIES, int SPLITS>
 __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4) ? 2 : 1) void attention_prefill_stream_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     T* __restrict__ out, int out_stride, const int* __restrict__ q_starts, const int* __restrict__ context_lens,
-    const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads, int page_shift, int window, float scale) {
+    const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads, int page_shift, int window, float scale, ScoreOptions options) {
     typedef Layout<T, HD, SPLITS> L;
     constexpr bool FP32 = L::FP32;
     constexpr int QSUB = QUERIES / 32;
@@ -332,6 +332,15 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
             const int sub_first_position = context + tile_q0 + qs * 32;
             const bool interior = window == 0 && tile_q0 + qs * 32 + 31 < q_len && k0 + KEYS - 1 <= sub_first_position;
             float tile_max = -INFINITY;
+            if (options.softcap > 0.0f) {   // a capped score, left divided by the scale as the plain ones are: cap tanh(scale s / cap) / scale
+                const float back = options.softcap / scale, into = scale / options.softcap;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    if constexpr (FP32) s_acc[qs][v] = back * tanhf(s_acc[qs][v] * into);
+                    else   // tanh x = 1 - 2 / (1 + e^(2x)), the hardware's 2^x and reciprocal: five instructions a score
+                        s_acc[qs][v] = __builtin_fmaf(-2.0f * back, __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(s_acc[qs][v] * (into * 2.8853900817779268f))), back);
+                }
+            }
             if (interior) {
 #pragma unroll
                 for (int v = 0; v < 16; v++) tile_max = fmaxf(tile_max, s_acc[qs][v]);
@@ -479,6 +488,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
             weight[w] = weight_of(stats_lds[w][qs * 32 + lane32][0] - best);  // a wave that saw no key: a weight of 0
             total += weight[w] * stats_lds[w][qs * 32 + lane32][1];
         }
+        if (options.sinks) total += weight_of(options.sinks[head] * (FP32 ? 1.0f : 1.4426950408889634f) - best);   // the sink: once, with no value
         const float inverse = 1.0f / total;
         T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * HD + i2 * 32;
 #pragma unroll
@@ -514,7 +524,7 @@ inline bool takes(int head_size, int page_size, int max_q_len, float scale, int 
 template <typename T, int HD, int QUERIES, int SPLITS>
 void launch_queries(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
                     const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int n_heads, int n_kv_heads,
-                    int page_shift, int window, float scale, hipStream_t stream) {
+                    int page_shift, int window, float scale, ScoreOptions options, hipStream_t stream) {
     constexpr int LDS_BYTES = Layout<T, HD, SPLITS>::LDS_BYTES;
     static bool raised = false;  // per instantiation: the limit on dynamic LDS is a property of the kernel
     if (!raised && LDS_BYTES > 60 * 1024)  // (if this fails the launch below fails too, and the entry point reports that)
@@ -524,16 +534,16 @@ void launch_queries(const void* q, int q_stride, const void* k_pages, const void
     mllm_count_kernel(MLLM_K_ATTENTION_PREFILL_STREAM);
     attention_prefill_stream_kernel<T, HD, QUERIES, SPLITS><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
         (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens,
-        block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);
+        block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, options);
 }
 
 template <typename T, int HD>
 void launch(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
             const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int max_len, int n_heads,
-            int n_kv_heads, int page_shift, int window, float scale, hipStream_t stream) {
+            int n_kv_heads, int page_shift, int window, float scale, ScoreOptions options, hipStream_t stream) {
 #define MLLM_STREAM_LAUNCH(QUERIES, SPLITS)                                                                                                 \
     launch_queries<T, HD, QUERIES, SPLITS>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, \
-                                           n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, stream)
+                                           n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, options, stream)
     if constexpr (sizeof(T) == 4) {
         // 32-bit: the matrix cores are what a wave waits for (a tile of 32 keys is 96 products of 64 cycles for 32 queries),
         // so blocks of 32 queries, which the compute units take in turn, the ones with the most keys first

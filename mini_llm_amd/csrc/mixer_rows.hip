@@ -50,35 +50,49 @@ __global__ __launch_bounds__(256) void projection_rows_kernel(const float* __res
         k_factor = 1.0f / sqrtf(block_sum(squares, scratch) / (float)k_width + eps);
     }
     const float position = (float)positions[row];
-    // one element of a normed, rotated head: d its place in the head, at the head's first element in the row
-    auto turned = [&](const float* in, const float* gain, float factor, int at, int d) -> float {
-        const float own = in[at + d] * factor * (gain ? gain[at + d] : 1.0f);
-        if (d >= rot_dims) return own;
-        const int e = d ^ 1;
-        const float other = in[at + e] * factor * (gain ? gain[at + e] : 1.0f);
-        const float angle = position * frequencies[d >> 1];
-        const float c = cosf(angle), s = sinf(angle);
-        return (d & 1) ? own * c + other * s : own * c - other * s;
+    // a pair of neighbouring elements of a normed head, rotated where it lies among the first rot_dims: d its first element's place
+    // in the head (even), `at` the head's first element in the row; elements beyond the head's own are zero
+    auto turned_pair = [&](const float* in, const float* gain, float factor, int at, int d, float& first, float& second) {
+        first = d < dim ? in[at + d] * factor * (gain ? gain[at + d] : 1.0f) : 0.0f;
+        second = d + 1 < dim ? in[at + d + 1] * factor * (gain ? gain[at + d + 1] : 1.0f) : 0.0f;
+        if (d < rot_dims) {
+            float s, c;
+            sincosf(position * frequencies[d >> 1], &s, &c);
+            const float u = first, w = second;
+            first = u * c - w * s;
+            second = w * c + u * s;
+        }
     };
-    for (int i = threadIdx.x; i < n_heads * head_size; i += blockDim.x) {
-        const int head = i / head_size, d = i % head_size;
-        q_out[(size_t)row * n_heads * head_size + i] = from_float<T>(d < dim ? turned(q_row, q_gain, q_factor, head * dim, d) : 0.0f);
+    const int half_head = head_size / 2;   // (heads in pages are multiples of 16 wide)
+    for (int i = threadIdx.x; i < n_heads * half_head; i += blockDim.x) {
+        const int head = i / half_head, d = 2 * (i % half_head);
+        float first, second;
+        turned_pair(q_row, q_gain, q_factor, head * dim, d, first, second);
+        T* to = q_out + (size_t)row * n_heads * head_size + (size_t)head * head_size + d;
+        to[0] = from_float<T>(first);
+        to[1] = from_float<T>(second);
     }
     if (!write_cache) return;
     const int slot = slots[row];
     if (slot < 0) return;
     const int page = slot / page_size, offset = slot % page_size;
     const float blend = v_other ? mix[0] : 0.0f;
-    for (int i = threadIdx.x; i < n_kv_heads * head_size; i += blockDim.x) {
-        const int head = i / head_size, d = i % head_size;
+    for (int i = threadIdx.x; i < n_kv_heads * half_head; i += blockDim.x) {
+        const int head = i / half_head, d = 2 * (i % half_head);
         const size_t at = (((size_t)page * n_kv_heads + head) * page_size + offset) * head_size + d;
-        k_pages[at] = from_float<T>(d < dim ? turned(k_row, k_gain, k_factor, head * dim, d) : 0.0f);
-        float value = 0.0f;
-        if (d < vdim) {
-            value = v[(size_t)row * v_stride + head * vdim + d];
-            if (v_other) value = (1.0f - blend) * value + blend * v_other[(size_t)row * v_other_stride + head * vdim + d];
+        float first, second;
+        turned_pair(k_row, k_gain, k_factor, head * dim, d, first, second);
+        k_pages[at] = from_float<T>(first);
+        k_pages[at + 1] = from_float<T>(second);
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            float value = 0.0f;
+            if (d + e < vdim) {
+                value = v[(size_t)row * v_stride + head * vdim + d + e];
+                if (v_other) value = (1.0f - blend) * value + blend * v_other[(size_t)row * v_other_stride + head * vdim + d + e];
+            }
+            v_pages[at + e] = from_float<T>(value);
         }
-        v_pages[at] = from_float<T>(value);
     }
 }
 
@@ -106,6 +120,27 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const float* __restrict
     if (item >= (long long)n_rows * groups) return;
     const int row = (int)(item / groups), first = (int)(item % groups) * group;
     const float* in = x + (size_t)row * x_stride + first;
+    if (group <= 4 * WAVE) {
+        // everything the wave needs asked for at once, so that it waits for memory once
+        float xs[4], ws[4], gs[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int d = min(lane + r * WAVE, group - 1);
+            xs[r] = in[d];
+            ws[r] = weight ? weight[first + d] : 1.0f;
+            gs[r] = gate ? gate[(size_t)row * gate_stride + first + d] : 0.0f;
+        }
+        float squares = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) squares += lane + r * WAVE < group ? xs[r] * xs[r] : 0.0f;
+        const float factor = scale / sqrtf(wave_sum(squares) / (float)group + eps);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int d = lane + r * WAVE;
+            if (d < group) out[(size_t)row * out_stride + first + d] = from_float<T>(xs[r] * factor * ws[r] * (gate ? sigmoid_f(gs[r]) : 1.0f));
+        }
+        return;
+    }
     float squares = 0.0f;
     for (int d = lane; d < group; d += WAVE) squares += in[d] * in[d];
     const float factor = scale / sqrtf(wave_sum(squares) / (float)group + eps);

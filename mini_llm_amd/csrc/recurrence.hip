@@ -236,3 +236,411 @@ MLLM_API int mllm_recurrence(int kind, const float* q, int q_stride, const float
 #undef RECURRENCE_ARGS
     return mllm_check_launch("recurrence");
 }
+
+// ------------------------------------------------------------------------------------------------------------------------
+// Long portions: the same recurrences chunk by chunk, so that the rows of a portion do not wait for each other.
+//
+// Inside a chunk of L rows (b_t the sum of the log decays up to row t, g_s the log input gate of row s, both 0-based inside the
+// chunk; the state S0, n0, m0 at the chunk's start):
+//     m_t = b_t + max(m0, max_{s<=t}(g_s - b_s))
+//     o_t = [exp(b_t + m0 - m_t) q_t^T S0 + sum_{s<=t} exp(b_t - b_s + g_s - m_t) (q_t . k_s) v_s] / (max(|nq_t|, exp(-m_t)) + 1e-6)
+//     nq_t = exp(b_t + m0 - m_t) q_t . n0 + sum_{s<=t} exp(b_t - b_s + g_s - m_t) (q_t . k_s)
+// and over the whole chunk, with B = b_(L-1) and mu = max_s(B - b_s + g_s),
+//     U = sum_s exp(B - b_s + g_s - mu) k_s v_s^T,  m' = max(B + m0, mu),  S' = exp(B + m0 - m') S0 + exp(mu - m') U   (n likewise),
+// which is what the row-by-row recurrence gives, in another order of sums. Without gates (a fixed decay) g = 0, m = 0 throughout.
+// Three kernels: (1) every chunk's U, its share of n, B and mu, all chunks at once; (2) per (request, head) the chunks in order,
+// a few multiply-adds an element: each chunk's U is replaced by the state at its start, and the request's slot gets the state at
+// the portion's end; (3) every chunk's outputs, all chunks at once. The sums b_t are taken in 64-bit, so that the difference of
+// two of them is exact to 32 bits however far the gates have closed.
+//
+// Scratch: one record of dim * vdim + dim + 4 floats per (chunk, head). Chunk c of request r, whose first row in the batch is
+// f, has the record f / L + r: no two chunks of a batch share one, and there are at most rows / L + requests of them.
+// ------------------------------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int CHUNK_THREADS = 512, CHUNK_WAVES = CHUNK_THREADS / WAVE, CHUNK_VT = 64;
+
+template <int L>
+struct ChunkShape {
+    static constexpr int DIM_MAX = 4096 / L;   // L = 64: heads up to 64 wide; 32: up to 128; 16: up to 256
+    static constexpr int RPW = L / CHUNK_WAVES;
+};
+
+__device__ __forceinline__ size_t chunk_record(int first_row, int chunk_rows, int request) { return (size_t)(first_row / chunk_rows + request); }
+
+__device__ __forceinline__ double lanes_prefix_sum(double v, int lane) {
+#pragma unroll
+    for (int offset = 1; offset < WAVE; offset <<= 1) {
+        const double other = __shfl_up(v, offset, WAVE);
+        if (lane >= offset) v += other;
+    }
+    return v;
+}
+__device__ __forceinline__ double lanes_prefix_max(double v, int lane) {
+#pragma unroll
+    for (int offset = 1; offset < WAVE; offset <<= 1) {
+        const double other = __shfl_up(v, offset, WAVE);
+        if (lane >= offset) v = fmax(v, other);
+    }
+    return v;
+}
+
+// The log decay and log input gate of a row (see the head of this file).
+template <int MODE>
+__device__ __forceinline__ void row_gates(const float* gate_in, const float* gate_forget, int gate_stride, float cap, float log_decay, size_t row,
+                                          int head, float& log_keep, float& log_take) {
+    if (MODE == GATED) {
+        float gi = gate_in[row * gate_stride + head], gf = gate_forget[row * gate_stride + head];
+        if (cap > 0.0f) gi = cap * tanhf(gi / cap), gf = cap * tanhf(gf / cap);
+        log_take = gi;
+        log_keep = log_sigmoid_f(gf);
+    } else {
+        log_take = 0.0f;
+        log_keep = log_decay;
+    }
+}
+
+template <int L, int MODE>
+__global__ __launch_bounds__(CHUNK_THREADS) void chunk_sums_kernel(const float* __restrict__ k, int k_stride, const float* __restrict__ v, int v_stride,
+                                                                   const float* __restrict__ gate_in, const float* __restrict__ gate_forget,
+                                                                   int gate_stride, float cap, const float* __restrict__ decay,
+                                                                   const int* __restrict__ q_starts, const int* __restrict__ state_slots,
+                                                                   float* __restrict__ scratch, int dim, int vdim, int tiles) {
+    constexpr int DIM_MAX = ChunkShape<L>::DIM_MAX;
+    __shared__ float Ks[L][DIM_MAX];
+    __shared__ float Vs[L][CHUNK_VT];
+    __shared__ float weight[L];
+    const int request = blockIdx.x, head = blockIdx.y, n_heads = gridDim.y, chunk = blockIdx.z / tiles, tile = blockIdx.z % tiles;
+    const int first_row = q_starts[request], rows = q_starts[request + 1] - first_row;
+    if (state_slots[request] < 0 || chunk * L >= rows) return;
+    const int n_valid = min(L, rows - chunk * L), chunk_first = first_row + chunk * L;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const size_t record_floats = (size_t)dim * vdim + dim + 4;
+    float* record = scratch + (chunk_record(chunk_first, L, request) * n_heads + head) * record_floats;
+
+    for (int e = tid; e < L * dim; e += CHUNK_THREADS) {
+        const int s = e / dim, i = e % dim;
+        float value = 0.0f;
+        if (s < n_valid) {
+            value = k[(size_t)(chunk_first + s) * k_stride + head * dim + i];
+            if (MODE == DECAYED) value = silu_f(value);
+        }
+        Ks[s][i] = value;
+    }
+    for (int e = tid; e < L * CHUNK_VT; e += CHUNK_THREADS) {
+        const int s = e / CHUNK_VT, c = tile * CHUNK_VT + e % CHUNK_VT;
+        float value = 0.0f;
+        if (s < n_valid && c < vdim) {
+            value = v[(size_t)(chunk_first + s) * v_stride + head * vdim + c];
+            if (MODE == DECAYED) value = silu_f(value);
+        }
+        Vs[s][e % CHUNK_VT] = value;
+    }
+    if (wave == 0) {
+        float log_keep = 0.0f, log_take = 0.0f;
+        if (lane < n_valid) row_gates<MODE>(gate_in, gate_forget, gate_stride, cap, MODE == DECAYED ? logf(decay[head]) : 0.0f, (size_t)(chunk_first + lane), head, log_keep, log_take);
+        const double b = lanes_prefix_sum((double)log_keep, lane);
+        const double total = __shfl(b, n_valid - 1, WAVE);
+        const double reach = lane < n_valid ? (total - b) + (double)log_take : -INFINITY;
+        const float mu = MODE == GATED ? wave_max((float)reach) : 0.0f;
+        if (lane < L) weight[lane] = lane < n_valid ? expf((float)(reach - (double)mu)) : 0.0f;
+        if (lane == 0 && tile == 0) {
+            record[record_floats - 4] = (float)total;
+            record[record_floats - 3] = mu;
+        }
+    }
+    __syncthreads();
+    // U[i][j] = sum_s weight_s k_s[i] v_s[j]: a lane a column of the tile, a wave every eighth row i
+    constexpr int ROWS = DIM_MAX / CHUNK_WAVES;
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+    for (int s = 0; s < n_valid; s++) {
+        const float vv = Vs[s][lane] * weight[s];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) acc[r] += Ks[s][wave + r * CHUNK_WAVES] * vv;
+    }
+    const int j = tile * CHUNK_VT + lane;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const int i = wave + r * CHUNK_WAVES;
+        if (i < dim && j < vdim) record[(size_t)i * vdim + j] = acc[r];
+    }
+    if (MODE == GATED && tile == 0 && tid < dim) {
+        float sum = 0.0f;
+        for (int s = 0; s < n_valid; s++) sum += weight[s] * Ks[s][tid];
+        record[(size_t)dim * vdim + tid] = sum;
+    }
+}
+
+// The chunks of one (request, head) in order. A block takes up to 4,096 elements of the matrix (16 a thread); the block of the
+// first elements also moves n and m on. Each chunk's record gets the state at the chunk's start (matrix, n, and m in its last
+// place but two), and the request's slot the state at the portion's end.
+template <int MODE>
+__global__ __launch_bounds__(256) void chunk_scan_kernel(const int* __restrict__ q_starts, const int* __restrict__ state_slots, float* __restrict__ scratch,
+                                                         float* __restrict__ state, long long state_stride, long long n_at, long long m_at, int dim, int vdim,
+                                                         int chunk_rows) {
+    constexpr int PER = 16;
+    const int request = blockIdx.x, head = blockIdx.y, n_heads = gridDim.y;
+    const int slot = state_slots[request];
+    const int first_row = q_starts[request], rows = q_starts[request + 1] - first_row;
+    if (slot < 0 || rows <= 0) return;
+    const int n_chunks = (rows + chunk_rows - 1) / chunk_rows;
+    const size_t elements = (size_t)dim * vdim, record_floats = elements + dim + 4;
+    const size_t base = (size_t)blockIdx.z * 256 * PER;
+    float* mine = state + (size_t)slot * state_stride;
+    float* S_at = mine + (size_t)head * elements;
+    const bool first_block = blockIdx.z == 0;
+    const int tid = threadIdx.x;
+    float S[PER], n = 0.0f;
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const size_t e = base + (size_t)u * 256 + tid;
+        S[u] = e < elements ? S_at[e] : 0.0f;
+    }
+    if (MODE == GATED && first_block && tid < dim) n = mine[n_at + (size_t)head * dim + tid];
+    float m = MODE == GATED ? mine[m_at + head] : 0.0f;
+    auto record_of = [&](int c) { return scratch + (chunk_record(first_row + c * chunk_rows, chunk_rows, request) * n_heads + head) * record_floats; };
+    // the next chunk's numbers are asked for before this chunk's are used
+    float next[PER], next_n = 0.0f, next_total, next_mu;
+    {
+        float* record = record_of(0);
+#pragma unroll
+        for (int u = 0; u < PER; u++) {
+            const size_t e = base + (size_t)u * 256 + tid;
+            next[u] = e < elements ? record[e] : 0.0f;
+        }
+        if (MODE == GATED && first_block && tid < dim) next_n = record[elements + tid];
+        next_total = record[record_floats - 4];
+        next_mu = record[record_floats - 3];
+    }
+    for (int c = 0; c < n_chunks; c++) {
+        float* record = record_of(c);
+        float sums[PER];
+#pragma unroll
+        for (int u = 0; u < PER; u++) sums[u] = next[u];
+        const float sum_n = next_n, total = next_total, mu = next_mu;
+        if (c + 1 < n_chunks) {
+            float* ahead = record_of(c + 1);
+#pragma unroll
+            for (int u = 0; u < PER; u++) {
+                const size_t e = base + (size_t)u * 256 + tid;
+                next[u] = e < elements ? ahead[e] : 0.0f;
+            }
+            if (MODE == GATED && first_block && tid < dim) next_n = ahead[elements + tid];
+            next_total = ahead[record_floats - 4];
+            next_mu = ahead[record_floats - 3];
+        }
+        float keep, take, m_new = 0.0f;
+        if (MODE == GATED) {
+            m_new = fmaxf(total + m, mu);
+            keep = expf(total + m - m_new);
+            take = expf(mu - m_new);
+        } else {
+            keep = expf(total);
+            take = 1.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < PER; u++) {
+            const size_t e = base + (size_t)u * 256 + tid;
+            if (e < elements) record[e] = S[u];
+            S[u] = keep * S[u] + take * sums[u];
+        }
+        if (MODE == GATED && first_block) {
+            if (tid < dim) {
+                record[elements + tid] = n;
+                n = keep * n + take * sum_n;
+            }
+            if (tid == 0) record[record_floats - 2] = m;
+        }
+        m = m_new;
+    }
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const size_t e = base + (size_t)u * 256 + tid;
+        if (e < elements) S_at[e] = S[u];
+    }
+    if (MODE == GATED && first_block) {
+        if (tid < dim) mine[n_at + (size_t)head * dim + tid] = n;
+        if (tid == 0) mine[m_at + head] = m;
+    }
+}
+
+template <int L, int MODE>
+__global__ __launch_bounds__(CHUNK_THREADS) void chunk_output_kernel(const float* __restrict__ q, int q_stride, const float* __restrict__ k, int k_stride,
+                                                                     const float* __restrict__ v, int v_stride, const float* __restrict__ gate_in,
+                                                                     const float* __restrict__ gate_forget, int gate_stride, float cap,
+                                                                     const float* __restrict__ decay, float q_scale, const int* __restrict__ q_starts,
+                                                                     const int* __restrict__ state_slots, const float* __restrict__ scratch,
+                                                                     float* __restrict__ out, int out_stride, int dim, int vdim, int tiles) {
+    constexpr int DIM_MAX = ChunkShape<L>::DIM_MAX, RPW = ChunkShape<L>::RPW;
+    __shared__ __align__(16) float Qs[L][DIM_MAX];
+    __shared__ float Kt[DIM_MAX][L];       // transposed; once the scores are taken, its first L rows hold them: A[t][s]
+    __shared__ float Vs[L][CHUNK_VT];
+    __shared__ double b_of[L];
+    __shared__ double m_of[L];
+    __shared__ float take_of[L], start_weight[L], nq_of[L];
+    const int request = blockIdx.x, head = blockIdx.y, n_heads = gridDim.y, chunk = blockIdx.z / tiles, tile = blockIdx.z % tiles;
+    const int first_row = q_starts[request], rows = q_starts[request + 1] - first_row;
+    if (state_slots[request] < 0 || chunk * L >= rows) return;
+    const int n_valid = min(L, rows - chunk * L), chunk_first = first_row + chunk * L;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const size_t elements = (size_t)dim * vdim, record_floats = elements + dim + 4;
+    const float* record = scratch + (chunk_record(chunk_first, L, request) * n_heads + head) * record_floats;
+
+    for (int e = tid; e < L * dim; e += CHUNK_THREADS) {
+        const int s = e / dim, i = e % dim;
+        float qv = 0.0f, kv = 0.0f;
+        if (s < n_valid) {
+            qv = q[(size_t)(chunk_first + s) * q_stride + head * dim + i];
+            kv = k[(size_t)(chunk_first + s) * k_stride + head * dim + i];
+            if (MODE == DECAYED) qv = silu_f(qv), kv = silu_f(kv);
+            qv *= q_scale;
+        }
+        Qs[s][i] = qv;
+        Kt[i][s] = kv;
+    }
+    for (int e = tid; e < L * CHUNK_VT; e += CHUNK_THREADS) {
+        const int s = e / CHUNK_VT, c = tile * CHUNK_VT + e % CHUNK_VT;
+        float value = 0.0f;
+        if (s < n_valid && c < vdim) {
+            value = v[(size_t)(chunk_first + s) * v_stride + head * vdim + c];
+            if (MODE == DECAYED) value = silu_f(value);
+        }
+        Vs[s][e % CHUNK_VT] = value;
+    }
+    if (wave == 0) {
+        float log_keep = 0.0f, log_take = 0.0f;
+        if (lane < n_valid) row_gates<MODE>(gate_in, gate_forget, gate_stride, cap, MODE == DECAYED ? logf(decay[head]) : 0.0f, (size_t)(chunk_first + lane), head, log_keep, log_take);
+        const double b = lanes_prefix_sum((double)log_keep, lane);
+        double m_row = 0.0, from_start = b;
+        if (MODE == GATED) {
+            const double m_start = (double)record[record_floats - 2];
+            const double best = lanes_prefix_max(lane < n_valid ? (double)log_take - b : -INFINITY, lane);
+            m_row = b + fmax(m_start, best);
+            from_start = b + m_start - m_row;
+        }
+        if (lane < L) {
+            b_of[lane] = b;
+            m_of[lane] = m_row;
+            take_of[lane] = log_take;
+            start_weight[lane] = expf((float)from_start);
+        }
+    }
+    __syncthreads();
+    // ---- scores: a lane a key s, a wave every eighth query t ----
+    float a[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; r++) a[r] = 0.0f;
+    if (lane < L) {
+        for (int i = 0; i < dim; i += 4) {
+            const float k0 = Kt[i][lane], k1 = Kt[i + 1][lane], k2 = Kt[i + 2][lane], k3 = Kt[i + 3][lane];
+#pragma unroll
+            for (int r = 0; r < RPW; r++) {
+                const f32x4 qq = *reinterpret_cast<const f32x4*>(&Qs[wave + r * CHUNK_WAVES][i]);
+                a[r] += qq[0] * k0 + qq[1] * k1 + qq[2] * k2 + qq[3] * k3;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            const int t = wave + r * CHUNK_WAVES;
+            const bool sees = lane <= t && t < n_valid;
+            a[r] = sees ? a[r] * expf((float)((b_of[t] - b_of[lane]) + (double)take_of[lane] - m_of[t])) : 0.0f;
+        }
+    }
+    __syncthreads();   // everybody has read the keys
+    float (*A)[L] = Kt;
+    const float* n_start = record + elements;
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        const int t = wave + r * CHUNK_WAVES;
+        if (lane < L) A[t][lane] = a[r];
+        if (MODE == GATED) {
+            float with_start = 0.0f;
+            for (int i = lane; i < dim; i += WAVE) with_start += Qs[t][i] * n_start[i];
+            const float nq = wave_sum(lane < L ? a[r] : 0.0f) + start_weight[t] * wave_sum(with_start);
+            if (lane == 0) nq_of[t] = nq;
+        }
+    }
+    __syncthreads();
+    // ---- outputs: a lane a column of the tile, a wave every eighth row ----
+    const int j = tile * CHUNK_VT + lane;
+    const int column = min(j, vdim - 1);
+    float inside[RPW], before[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; r++) inside[r] = before[r] = 0.0f;
+    for (int s = 0; s < n_valid; s++) {
+        const float vv = Vs[s][lane];
+#pragma unroll
+        for (int r = 0; r < RPW; r++) inside[r] += A[wave + r * CHUNK_WAVES][s] * vv;
+    }
+    for (int i = 0; i < dim; i++) {
+        const float sv = record[(size_t)i * vdim + column];
+#pragma unroll
+        for (int r = 0; r < RPW; r++) before[r] += Qs[wave + r * CHUNK_WAVES][i] * sv;
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        const int t = wave + r * CHUNK_WAVES;
+        if (t >= n_valid || j >= vdim) continue;
+        float value = inside[r] + start_weight[t] * before[r];
+        if (MODE == GATED) value /= fmaxf(fabsf(nq_of[t]), expf((float)-m_of[t])) + 1e-6f;
+        out[(size_t)(chunk_first + t) * out_stride + head * vdim + j] = value;
+    }
+}
+
+int chunk_rows_for(int dim) { return dim <= 64 ? 64 : (dim <= 128 ? 32 : 16); }
+
+}  // namespace
+
+// The rows a chunk holds for heads of `dim` (0: the chunked kernels do not take such heads).
+MLLM_API int mllm_recurrence_chunk_rows(int dim) { return dim >= 4 && dim <= 256 && dim % 4 == 0 ? chunk_rows_for(dim) : 0; }
+
+// The same as mllm_recurrence for batches with long portions: max_rows is the longest portion of the batch (or a bound on it),
+// scratch holds (n_rows / chunk rows + n_requests + 1) * n_heads * (dim * vdim + dim + 4) floats.
+MLLM_API int mllm_recurrence_chunked(int kind, const float* q, int q_stride, const float* k, int k_stride, const float* v, int v_stride, const float* gate_in,
+                                     const float* gate_forget, int gate_stride, float cap, const float* decay, float q_scale, float* state,
+                                     long long state_stride, long long n_at, long long m_at, const int* q_starts, const int* state_slots, float* out,
+                                     int out_stride, int n_requests, int n_heads, int dim, int vdim, int max_rows, float* scratch, long long scratch_floats,
+                                     int n_rows, hipStream_t stream) {
+    MLLM_REQUIRE(kind == GATED || kind == DECAYED, "recurrence_chunked: unknown kind %d", kind);
+    MLLM_REQUIRE(n_requests >= 0 && n_heads > 0 && vdim > 0 && max_rows >= 0 && n_rows >= 0, "recurrence_chunked: bad sizes");
+    MLLM_REQUIRE(mllm_recurrence_chunk_rows(dim) > 0, "recurrence_chunked: heads of %d are not taken (a multiple of 4 up to 256)", dim);
+    MLLM_REQUIRE(q_stride >= n_heads * dim && k_stride >= n_heads * dim && v_stride >= n_heads * vdim && out_stride >= n_heads * vdim, "recurrence_chunked: rows are too short for the heads");
+    MLLM_REQUIRE(q != nullptr && k != nullptr && v != nullptr && state != nullptr && q_starts != nullptr && state_slots != nullptr && out != nullptr && scratch != nullptr, "recurrence_chunked: a missing operand");
+    const long long matrices = (long long)n_heads * dim * vdim;
+    if (kind == GATED) {
+        MLLM_REQUIRE(gate_in != nullptr && gate_forget != nullptr && gate_stride >= n_heads, "recurrence_chunked: the gates are missing");
+        MLLM_REQUIRE(n_at >= matrices && m_at >= n_at + (long long)n_heads * dim && state_stride >= m_at + n_heads, "recurrence_chunked: the state's parts overlap");
+    } else {
+        MLLM_REQUIRE(decay != nullptr && state_stride >= matrices, "recurrence_chunked: the decays are missing or the state is too small");
+    }
+    const int L = chunk_rows_for(dim);
+    MLLM_REQUIRE(scratch_floats >= ((long long)n_rows / L + n_requests + 1) * n_heads * ((long long)dim * vdim + dim + 4), "recurrence_chunked: the scratch memory is too small");
+    if (n_requests == 0 || max_rows == 0) return 0;
+    const int tiles = ceil_div(vdim, CHUNK_VT), chunks = ceil_div(max_rows, L);
+    MLLM_REQUIRE((long long)chunks * tiles <= 65535, "recurrence_chunked: too many chunks for one launch");
+    dim3 grid(n_requests, n_heads, chunks * tiles), scan_grid(n_requests, n_heads, ceil_div(dim * vdim, 4096));
+#define CHUNKED(LL, MODE)                                                                                                                              \
+    do {                                                                                                                                               \
+        mllm_count_kernel(MLLM_K_RECURRENCE);                                                                                                          \
+        chunk_sums_kernel<LL, MODE><<<grid, CHUNK_THREADS, 0, stream>>>(k, k_stride, v, v_stride, gate_in, gate_forget, gate_stride, cap, decay, q_starts, \
+                                                                        state_slots, scratch, dim, vdim, tiles);                                       \
+        mllm_count_kernel(MLLM_K_RECURRENCE);                                                                                                          \
+        chunk_scan_kernel<MODE><<<scan_grid, 256, 0, stream>>>(q_starts, state_slots, scratch, state, state_stride, n_at, m_at, dim, vdim, LL);         \
+        mllm_count_kernel(MLLM_K_RECURRENCE);                                                                                                          \
+        chunk_output_kernel<LL, MODE><<<grid, CHUNK_THREADS, 0, stream>>>(q, q_stride, k, k_stride, v, v_stride, gate_in, gate_forget, gate_stride, cap, \
+                                                                          decay, q_scale, q_starts, state_slots, scratch, out, out_stride, dim, vdim, tiles); \
+    } while (0)
+    if (kind == GATED) {
+        if (L == 64) CHUNKED(64, GATED);
+        else if (L == 32) CHUNKED(32, GATED);
+        else CHUNKED(16, GATED);
+    } else {
+        if (L == 64) CHUNKED(64, DECAYED);
+        else if (L == 32) CHUNKED(32, DECAYED);
+        else CHUNKED(16, DECAYED);
+    }
+#undef CHUNKED
+    return mllm_check_launch("recurrence_chunked");
+}

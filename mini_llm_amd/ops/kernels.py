@@ -1112,14 +1112,20 @@ def recurrence_supported(dim: int, vdim: int) -> bool:
     return bool(library().mllm_recurrence_supported(int(dim), int(vdim)))
 
 
+RECURRENCE_ROW_BY_ROW = 8   # batches whose longest portion has at most so many rows walk them row by row; longer ones go chunk by chunk
+
+
 def recurrence(q, k, v, state, q_starts, state_slots, n_heads, dim, vdim, *, gate_in=None, gate_forget=None, cap: float = 0.0, decay=None,
-               q_scale: float = 1.0):
+               q_scale: float = 1.0, max_q_len: int | None = None, positive_decay: bool = True):
     """A matrix per head and request, moved on row by row: S <- a S + b k v^T, o = S^T q, all in 32-bit. q, k: float32 [rows, n_heads *
     dim]; v: [rows, n_heads * vdim] (strided views); ``state``: float32 [slots, >= what the kind keeps] (rows may be strided);
     the rows of request r are q_starts[r] .. q_starts[r + 1], its state in slot state_slots[r] (negative: skipped).
     With ``gate_in`` / ``gate_forget`` (float32 [rows, n_heads], the sums of the gates' projections): the matrix memory of an mLSTM, the
     gates capped at +-cap (0: not), a normaliser and a running maximum kept behind the matrices ([heads, dim, vdim], [heads, dim],
-    [heads]). With ``decay`` (float32 [n_heads]): a = decay_h, b = 1, and q, k, v go through silu. Returns o, float32 [rows, n_heads * vdim]."""
+    [heads]). With ``decay`` (float32 [n_heads]): a = decay_h, b = 1, and q, k, v go through silu. Returns o, float32 [rows, n_heads * vdim].
+    ``max_q_len``: the longest portion of the batch, or a bound on it; above RECURRENCE_ROW_BY_ROW the portions run chunk by chunk (all
+    chunks of all requests at once, a short pass over the chunks in order between), which gives the same sums in another order.
+    ``positive_decay`` False (a decay of zero, whose logarithm the chunks would need) keeps the batch row by row."""
     _rows_f32(q, "q", n_heads * dim)
     _rows_f32(k, "k", n_heads * dim)
     _rows_f32(v, "v", n_heads * vdim)
@@ -1141,6 +1147,14 @@ def recurrence(q, k, v, state, q_starts, state_slots, n_heads, dim, vdim, *, gat
         _device_tensor(decay, "decay", torch.float32, 1)
         _require(decay.shape[0] == n_heads and state.shape[1] >= matrices, "one decay a head, and a state that holds the matrices")
     out = torch.empty((n, n_heads * vdim), dtype=torch.float32, device=q.device)
+    chunk_rows = library().mllm_recurrence_chunk_rows(dim) if max_q_len is not None and max_q_len > RECURRENCE_ROW_BY_ROW and positive_decay else 0
+    if chunk_rows:
+        scratch = torch.empty(((n // chunk_rows + n_requests + 1) * n_heads * (dim * vdim + dim + 4),), dtype=torch.float32, device=q.device)
+        check(library().mllm_recurrence_chunked(0 if gated else 1, _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), _ptr(gate_forget),
+                                                gate_in.stride(0) if gated else 0, float(cap or 0.0), _ptr(decay), float(q_scale), _ptr(state), state.stride(0), matrices,
+                                                matrices + n_heads * dim, _ptr(q_starts), _ptr(state_slots), _ptr(out), out.stride(0), n_requests, n_heads, dim, vdim,
+                                                int(max_q_len), _ptr(scratch), scratch.numel(), n, _stream()))
+        return out
     check(library().mllm_recurrence(0 if gated else 1, _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), _ptr(gate_forget),
                                     gate_in.stride(0) if gated else 0, float(cap or 0.0), _ptr(decay), float(q_scale), _ptr(state), state.stride(0), matrices,
                                     matrices + n_heads * dim, _ptr(q_starts), _ptr(state_slots), _ptr(out), out.stride(0), n_requests, n_heads, dim, vdim, _stream()))

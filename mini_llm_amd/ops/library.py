@@ -66,6 +66,9 @@ _SIGNATURES = {
     "mllm_recurrence_supported": [c_int, c_int],
     "mllm_recurrence": [c_int, P, c_int, P, c_int, P, c_int, P, P, c_int, c_float, P, c_float, P, c_longlong, c_longlong, c_longlong, P, P, P, c_int, c_int,
                         c_int, c_int, c_int, P],
+    "mllm_recurrence_chunk_rows": [c_int],
+    "mllm_recurrence_chunked": [c_int, P, c_int, P, c_int, P, c_int, P, P, c_int, c_float, P, c_float, P, c_longlong, c_longlong, c_longlong, P, P, P, c_int,
+                                c_int, c_int, c_int, c_int, c_int, P, c_longlong, c_int, P],
 }
 
 

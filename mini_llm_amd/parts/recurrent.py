@@ -83,7 +83,7 @@ class MatrixMemoryMixer(Mixer):
         at = 2 * qw + 2 * vw
         summed = kernels.recurrence(q, k, v, ctx.state, batch.q_starts, batch.state_slots, H, self.dim, self.vdim,
                                     gate_in=fused[:, at : at + H], gate_forget=fused[:, at + H : at + 2 * H], cap=self.gate_cap or 0.0,
-                                    q_scale=self.dim ** -0.5)
+                                    q_scale=self.dim ** -0.5, max_q_len=batch.max_q_len)
         mixed = torch.empty((x.shape[0], vw), dtype=x.dtype, device=x.device)
         kernels.gated_norm(summed, self.norm, gate, self.eps, mixed, group=self.vdim, scale=self.out_scale)
         return self._out_product(mixed, self.o, residual)
@@ -129,7 +129,8 @@ class DecayedLinearAttention(Mixer):
         fused = kernels.linear(x, self.w_in, out_dtype=torch.float32)
         qw, vw = H * self.dim, H * self.vdim
         q, k, v, gate = fused[:, :qw], fused[:, qw : 2 * qw], fused[:, 2 * qw : 2 * qw + vw], fused[:, 2 * qw + vw :]
-        summed = kernels.recurrence(q, k, v, ctx.state, batch.q_starts, batch.state_slots, H, self.dim, self.vdim, decay=self.decay)
+        summed = kernels.recurrence(q, k, v, ctx.state, batch.q_starts, batch.state_slots, H, self.dim, self.vdim, decay=self.decay,
+                                    max_q_len=batch.max_q_len, positive_decay=min(self.decay_values) > 0)
         mixed = torch.empty((x.shape[0], vw), dtype=x.dtype, device=x.device)
         kernels.gated_norm(summed, self.norm, gate, self.eps, mixed, scale=self.out_scale)
         return self._out_product(mixed, self.o, residual)

@@ -202,8 +202,9 @@ def step_through(run, lengths, sizes, n_slots=6):
     return [np.concatenate(g) for g in got]
 
 
+@pytest.mark.parametrize("chunked", [False, True])
 @pytest.mark.parametrize("heads,dim,vdim", SIZES)
-def test_matrix_memory_in_portions_against_token_by_token(heads, dim, vdim):
+def test_matrix_memory_in_portions_against_token_by_token(heads, dim, vdim, chunked):
     k = kernels()
     assert k.recurrence_supported(dim, vdim)
     rng = np.random.default_rng(dim * vdim)
@@ -229,7 +230,7 @@ def test_matrix_memory_in_portions_against_token_by_token(heads, dim, vdim):
         qw, vw = heads * dim, heads * vdim
         return k.recurrence(fused[:, :qw], fused[:, qw : 2 * qw], fused[:, 2 * qw : 2 * qw + vw], state[:, :size], starts, slots, heads, dim, vdim,
                             gate_in=fused[:, 2 * qw + vw : 2 * qw + vw + heads], gate_forget=fused[:, 2 * qw + vw + heads :], cap=cap,
-                            q_scale=dim ** -0.5).cpu().numpy()
+                            q_scale=dim ** -0.5, max_q_len=max(n for _, _, n in parts) + 8 if chunked else None).cpu().numpy()
 
     got = step_through(run, lengths, sizes=(7, 2, 16, 3, 9, 64))
     for a, b in zip(got, want):
@@ -237,8 +238,9 @@ def test_matrix_memory_in_portions_against_token_by_token(heads, dim, vdim):
     assert (state[2] == 5.0).all() and (state[5] == 0).all() and (state[:, size:][[0, 1, 3, 4]] == 0).all()
 
 
+@pytest.mark.parametrize("chunked", [False, True])
 @pytest.mark.parametrize("heads,dim,vdim", SIZES)
-def test_decayed_recurrence_in_portions_against_token_by_token(heads, dim, vdim):
+def test_decayed_recurrence_in_portions_against_token_by_token(heads, dim, vdim, chunked):
     k = kernels()
     rng = np.random.default_rng(dim + vdim)
     lengths = [70, 19, 33]
@@ -251,9 +253,10 @@ def test_decayed_recurrence_in_portions_against_token_by_token(heads, dim, vdim)
 
     def run(parts, starts, slots):
         rows = [gpu(np.concatenate([data[i][j][at : at + n] for i, at, n in parts])) for j in range(3)]
-        return k.recurrence(rows[0], rows[1], rows[2], state, starts, slots, heads, dim, vdim, decay=gpu(decay)).cpu().numpy()
+        return k.recurrence(rows[0], rows[1], rows[2], state, starts, slots, heads, dim, vdim, decay=gpu(decay),
+                            max_q_len=max(n for _, _, n in parts) + 8 if chunked else None).cpu().numpy()
 
-    got = step_through(run, lengths, sizes=(5, 2, 31, 8))
+    got = step_through(run, lengths, sizes=(5, 2, 31, 8, 70))
     for a, b in zip(got, want):
         np.testing.assert_allclose(a, b, atol=2e-4, rtol=2e-4)
 
@@ -271,13 +274,14 @@ def test_matrix_memory_keeps_a_token_from_hundreds_of_steps_back():
     gi[3] = 5.0
     want = plain.mlstm_recurrence(q.reshape(n, 1, dim), kk.reshape(n, 1, dim), v.reshape(n, 1, vdim), gi, plain.log_sigmoid(gf)).reshape(n, vdim)
     assert np.allclose(want[-1], v[3] * np.sign(key @ key), atol=1e-3)
-    for cut in (n, 1, 64):
+    for cut in (n, 1, 64, -n, -100):   # (negative: chunk by chunk)
         state = torch.zeros((1, dim * vdim + dim + 1)).cuda()
         got = []
+        chunked, cut = cut < 0, abs(cut)
         for at in range(0, n, cut):
             m = min(cut, n - at)
             got.append(k.recurrence(gpu(q[at : at + m]), gpu(kk[at : at + m]), gpu(v[at : at + m]), state, ints([0, m]), ints([0]), 1, dim, vdim,
-                                    gate_in=gpu(gi[at : at + m]), gate_forget=gpu(gf[at : at + m])).cpu().numpy())
+                                    gate_in=gpu(gi[at : at + m]), gate_forget=gpu(gf[at : at + m]), max_q_len=m if chunked else None).cpu().numpy())
             if cut == 1 and at > 40:
                 break
         got = np.concatenate(got)
