@@ -30,8 +30,8 @@ def _section(raw: dict, key: str, where: str, optional: bool = False):
 
 def recurrence_fits(dim: int, vdim: int) -> bool:
     """Whether the recurrence kernel takes heads of dim x vdim: a block holds tiles of up to 64 value columns, up to 512 / tile
-    parts along dim and up to 32 rows of the matrix a thread."""
-    return 1 <= dim <= 32 * max(1, min(dim, 512 // min(vdim, 64))) and vdim >= 1
+    parts along dim and up to 64 rows of the matrix a thread."""
+    return 1 <= dim <= 64 * max(1, min(dim, 512 // min(vdim, 64))) and vdim >= 1
 
 
 @dataclass(frozen=True)

@@ -167,7 +167,7 @@ struct Plan {
 };
 
 // How a head of dim x vdim is laid over a block: tiles of up to 64 value columns, as many parts along dim as 512 threads
-// allow, a power of two of rows of S a thread.
+// allow, a power of two of rows of S a thread (up to 64: two waves a SIMD leave a thread 256 registers).
 bool plan_for(int dim, int vdim, Plan& plan) {
     plan.VT = vdim <= 64 ? vdim : 64;
     plan.tiles = ceil_div(vdim, plan.VT);
@@ -176,7 +176,7 @@ bool plan_for(int dim, int vdim, Plan& plan) {
     if (most_parts < 1) most_parts = 1;
     plan.R = 1;
     while (plan.R * most_parts < dim) plan.R *= 2;
-    if (plan.R > 32) return false;
+    if (plan.R > 64) return false;
     plan.P = ceil_div(dim, plan.R);
     plan.threads = ceil_div(plan.P * plan.VT, 64) * 64;
     plan.TB = 8;
@@ -230,7 +230,8 @@ MLLM_API int mllm_recurrence(int kind, const float* q, int q_stride, const float
         case 4: LAUNCH(4); break;
         case 8: LAUNCH(8); break;
         case 16: LAUNCH(16); break;
-        default: LAUNCH(32); break;
+        case 32: LAUNCH(32); break;
+        default: LAUNCH(64); break;
     }
 #undef LAUNCH
 #undef RECURRENCE_ARGS

@@ -177,7 +177,7 @@ def test_gates_of_heads_and_of_elements():
     np.testing.assert_allclose(out.cpu().numpy(), plain.rms_unit(x.reshape(5, 2, 45), 1e-5).reshape(5, 90), atol=2e-5, rtol=2e-5)
 
 
-SIZES = [(2, 16, 24), (3, 8, 8), (1, 64, 64), (2, 48, 48), (2, 16, 130), (1, 128, 128), (4, 20, 12), (1, 256, 64), (2, 1, 1)]
+SIZES = [(2, 16, 24), (3, 8, 8), (1, 64, 64), (2, 48, 48), (2, 16, 130), (1, 128, 128), (4, 20, 12), (1, 256, 64), (2, 1, 1), (1, 384, 70)]
 
 
 def step_through(run, lengths, sizes, n_slots=6):
