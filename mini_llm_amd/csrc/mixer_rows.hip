@@ -33,23 +33,35 @@ __global__ __launch_bounds__(256) void projection_rows_kernel(const float* __res
                                                               int rot_dims, const int* __restrict__ positions, const int* __restrict__ slots,
                                                               T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages, int n_heads,
                                                               int n_kv_heads, int dim, int vdim, int head_size, int page_size, int write_cache) {
-    __shared__ float scratch[16];
+    __shared__ float scratch[2][16];
     const int row = blockIdx.x;
     const float* q_row = q + (size_t)row * q_stride;
     const float* k_row = k + (size_t)row * k_stride;
     const int q_width = n_heads * dim, k_width = n_kv_heads * dim;
-    float q_factor = 1.0f, k_factor = 1.0f;
-    if (q_gain) {
-        float squares = 0.0f;
-        for (int i = threadIdx.x; i < q_width; i += blockDim.x) squares += q_row[i] * q_row[i];
-        q_factor = 1.0f / sqrtf(block_sum(squares, scratch) / (float)q_width + eps);
+    // the row's position and slot are asked for together with its first elements, and both sums of squares settle in one exchange
+    const int position_of_row = positions[row];
+    const int slot = write_cache ? slots[row] : -1;
+    const float blend = v_other ? mix[0] : 0.0f;
+    float q_squares = 0.0f, k_squares = 0.0f;
+    if (q_gain)
+        for (int i = threadIdx.x; i < q_width; i += blockDim.x) q_squares += q_row[i] * q_row[i];
+    if (k_gain)
+        for (int i = threadIdx.x; i < k_width; i += blockDim.x) k_squares += k_row[i] * k_row[i];
+    q_squares = wave_sum(q_squares);
+    k_squares = wave_sum(k_squares);
+    if (threadIdx.x % WAVE == 0) {
+        scratch[0][threadIdx.x / WAVE] = q_squares;
+        scratch[1][threadIdx.x / WAVE] = k_squares;
     }
-    if (k_gain) {
-        float squares = 0.0f;
-        for (int i = threadIdx.x; i < k_width; i += blockDim.x) squares += k_row[i] * k_row[i];
-        k_factor = 1.0f / sqrtf(block_sum(squares, scratch) / (float)k_width + eps);
+    __syncthreads();
+    q_squares = k_squares = 0.0f;
+    for (int w = 0; w < (int)blockDim.x / WAVE; w++) {
+        q_squares += scratch[0][w];
+        k_squares += scratch[1][w];
     }
-    const float position = (float)positions[row];
+    const float q_factor = q_gain ? 1.0f / sqrtf(q_squares / (float)q_width + eps) : 1.0f;
+    const float k_factor = k_gain ? 1.0f / sqrtf(k_squares / (float)k_width + eps) : 1.0f;
+    const float position = (float)position_of_row;
     // a pair of neighbouring elements of a normed head, rotated where it lies among the first rot_dims: d its first element's place
     // in the head (even), `at` the head's first element in the row; elements beyond the head's own are zero
     auto turned_pair = [&](const float* in, const float* gain, float factor, int at, int d, float& first, float& second) {
@@ -72,11 +84,8 @@ __global__ __launch_bounds__(256) void projection_rows_kernel(const float* __res
         to[0] = from_float<T>(first);
         to[1] = from_float<T>(second);
     }
-    if (!write_cache) return;
-    const int slot = slots[row];
-    if (slot < 0) return;
+    if (slot < 0) return;   // no cache write, or a padding row
     const int page = slot / page_size, offset = slot % page_size;
-    const float blend = v_other ? mix[0] : 0.0f;
     for (int i = threadIdx.x; i < n_kv_heads * half_head; i += blockDim.x) {
         const int head = i / half_head, d = 2 * (i % half_head);
         const size_t at = (((size_t)page * n_kv_heads + head) * page_size + offset) * head_size + d;
@@ -145,6 +154,48 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const float* __restrict
     for (int d = lane; d < group; d += WAVE) squares += in[d] * in[d];
     const float factor = scale / sqrtf(wave_sum(squares) / (float)group + eps);
     for (int d = lane; d < group; d += WAVE) {
+        float value = in[d] * factor;
+        if (weight) value *= weight[first + d];
+        if (gate) value *= sigmoid_f(gate[(size_t)row * gate_stride + first + d]);
+        out[(size_t)row * out_stride + first + d] = from_float<T>(value);
+    }
+}
+
+// The same for wide groups, a block per (row, group): up to eight elements a thread stay in registers between the sum of squares
+// and the output, asked for at once with their gains and gates; wider groups are read again.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_norm_wide_kernel(const float* __restrict__ x, int x_stride, const float* __restrict__ weight,
+                                                              const float* __restrict__ gate, int gate_stride, float eps, float scale,
+                                                              T* __restrict__ out, int out_stride, int width, int group) {
+    __shared__ float scratch[16];
+    const int groups = width / group;
+    const int row = blockIdx.x / groups, first = (blockIdx.x % groups) * group;
+    const float* in = x + (size_t)row * x_stride + first;
+    constexpr int REGS = 8;
+    if (group <= REGS * 256) {
+        float xs[REGS], ws[REGS], gs[REGS];
+#pragma unroll
+        for (int r = 0; r < REGS; r++) {
+            const int d = min((int)threadIdx.x + r * 256, group - 1);
+            xs[r] = in[d];
+            ws[r] = weight ? weight[first + d] : 1.0f;
+            gs[r] = gate ? gate[(size_t)row * gate_stride + first + d] : 0.0f;
+        }
+        float squares = 0.0f;
+#pragma unroll
+        for (int r = 0; r < REGS; r++) squares += (int)threadIdx.x + r * 256 < group ? xs[r] * xs[r] : 0.0f;
+        const float factor = scale / sqrtf(block_sum(squares, scratch) / (float)group + eps);
+#pragma unroll
+        for (int r = 0; r < REGS; r++) {
+            const int d = threadIdx.x + r * 256;
+            if (d < group) out[(size_t)row * out_stride + first + d] = from_float<T>(xs[r] * factor * ws[r] * (gate ? sigmoid_f(gs[r]) : 1.0f));
+        }
+        return;
+    }
+    float squares = 0.0f;
+    for (int d = threadIdx.x; d < group; d += 256) squares += in[d] * in[d];
+    const float factor = scale / sqrtf(block_sum(squares, scratch) / (float)group + eps);
+    for (int d = threadIdx.x; d < group; d += 256) {
         float value = in[d] * factor;
         if (weight) value *= weight[first + d];
         if (gate) value *= sigmoid_f(gate[(size_t)row * gate_stride + first + d]);
@@ -249,6 +300,13 @@ MLLM_API int mllm_gated_norm(const float* x, int x_stride, const float* weight, 
     const long long items = (long long)n_rows * (width / group);
     const int blocks = (int)((items + 3) / 4);
     mllm_count_kernel(MLLM_K_GATED_NORM);
+    if (group > 4 * WAVE) {   // wide groups: a block each
+        MLLM_REQUIRE(items <= 0x7fffffffLL, "gated_norm: too many groups for one launch");
+        if (dtype == MLLM_F32) gated_norm_wide_kernel<float><<<(int)items, 256, 0, stream>>>(x, x_stride, weight, gate, gate_stride, eps, scale, (float*)out, out_stride, width, group);
+        else if (dtype == MLLM_BF16) gated_norm_wide_kernel<bf16_t><<<(int)items, 256, 0, stream>>>(x, x_stride, weight, gate, gate_stride, eps, scale, (bf16_t*)out, out_stride, width, group);
+        else MLLM_REQUIRE(false, "gated_norm: unknown dtype %d", dtype);
+        return mllm_check_launch("gated_norm");
+    }
     if (dtype == MLLM_F32) gated_norm_kernel<float><<<blocks, 256, 0, stream>>>(x, x_stride, weight, gate, gate_stride, eps, scale, (float*)out, out_stride, n_rows, width, group);
     else if (dtype == MLLM_BF16) gated_norm_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, x_stride, weight, gate, gate_stride, eps, scale, (bf16_t*)out, out_stride, n_rows, width, group);
     else MLLM_REQUIRE(false, "gated_norm: unknown dtype %d", dtype);

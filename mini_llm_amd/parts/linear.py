@@ -81,3 +81,16 @@ class BranchProduct:
             if k_blocks > 1:
                 return kernels.linear_split(x, weight, k_blocks)
         return kernels.linear(x, weight, bias, residual=residual, out_dtype=torch.float32)
+
+
+def fuse_rows(matrices, multiple: int = 16):
+    """The matrices of several products over the same input laid behind each other ([out, in] each), zero rows added up to a multiple
+    of ``multiple`` outputs: the products of many rows stream only matrices whose outputs are a multiple of 8, and the ones of few
+    rows take 16 outputs a block. The caller reads the columns it knows of the fused product and leaves the rest alone."""
+    import torch
+
+    fused = torch.cat(list(matrices), dim=0)
+    spare = -fused.shape[0] % multiple
+    if spare:
+        fused = torch.cat([fused, torch.zeros((spare, fused.shape[1]), dtype=fused.dtype, device=fused.device)], dim=0)
+    return fused.contiguous()

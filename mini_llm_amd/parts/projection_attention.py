@@ -24,7 +24,7 @@ from ..ops import kernels
 from ..weights.spec import TABLE, VECTOR, Normal, TensorSpec
 from .attention import MAX_HEAD_SIZE
 from .base import KVNeed, LayerContext, Mixer, StateNeed, register_part
-from .linear import BranchProduct
+from .linear import BranchProduct, fuse_rows
 from .positions import RotaryEncoding
 
 
@@ -86,7 +86,7 @@ class ProjectionNormAttention(Mixer):
         return specs
 
     def bind(self, tensors):
-        fused = torch.cat([tensors[name] for name in ("q", "k", "v", "g") if name in tensors], dim=0).contiguous()
+        fused = fuse_rows([tensors[name] for name in ("q", "k", "v", "g") if name in tensors])
         o = tensors["o"]
         if self.head_size != self.vdim:   # the attention leaves heads of head_size: the columns beyond a head's vdim meet zeros
             wide = torch.zeros((self.width, self.n_heads, self.head_size), dtype=o.dtype, device=o.device)

@@ -27,7 +27,7 @@ import torch
 from ..ops import kernels
 from ..weights.spec import TABLE, VECTOR, Normal, TensorSpec
 from .base import LayerContext, Mixer, StateNeed, register_part
-from .linear import BranchProduct
+from .linear import BranchProduct, fuse_rows
 
 
 def _whole_batch(batch) -> None:
@@ -60,12 +60,13 @@ class MatrixMemoryMixer(Mixer):
 
     def bind(self, tensors):
         H = self.n_heads
-        fused = torch.cat([tensors[name] for name in ("q", "k", "v", "g", "i", "f")], dim=0).contiguous()
+        fused = fuse_rows([tensors[name] for name in ("q", "k", "v", "g", "i", "f")])
         on_gpu = fused.is_cuda
         self.w_in = kernels.pack_matrix(fused) if on_gpu else fused
         self.b_in = torch.zeros((fused.shape[0],), dtype=torch.float32, device=fused.device)
-        self.b_in[-2 * H : -H] = tensors["i.b"]
-        self.b_in[-H:] = tensors["f.b"]
+        at = 2 * H * self.dim + 2 * H * self.vdim
+        self.b_in[at : at + H] = tensors["i.b"]
+        self.b_in[at + H : at + 2 * H] = tensors["f.b"]
         self.o = kernels.pack_matrix(tensors["o"].contiguous()) if on_gpu else tensors["o"]
         self.norm = tensors["norm"]
 
@@ -112,7 +113,7 @@ class DecayedLinearAttention(Mixer):
                 "o": TensorSpec((self.width, H * self.vdim), TABLE, Normal((H * self.vdim) ** -0.5))}
 
     def bind(self, tensors):
-        fused = torch.cat([tensors[name] for name in ("q", "k", "v", "g")], dim=0).contiguous()
+        fused = fuse_rows([tensors[name] for name in ("q", "k", "v", "g")])
         on_gpu = fused.is_cuda
         self.w_in = kernels.pack_matrix(fused) if on_gpu else fused
         self.o = kernels.pack_matrix(tensors["o"].contiguous()) if on_gpu else tensors["o"]
@@ -128,7 +129,7 @@ class DecayedLinearAttention(Mixer):
         _whole_batch(batch)
         fused = kernels.linear(x, self.w_in, out_dtype=torch.float32)
         qw, vw = H * self.dim, H * self.vdim
-        q, k, v, gate = fused[:, :qw], fused[:, qw : 2 * qw], fused[:, 2 * qw : 2 * qw + vw], fused[:, 2 * qw + vw :]
+        q, k, v, gate = fused[:, :qw], fused[:, qw : 2 * qw], fused[:, 2 * qw : 2 * qw + vw], fused[:, 2 * qw + vw : 2 * qw + 2 * vw]
         summed = kernels.recurrence(q, k, v, ctx.state, batch.q_starts, batch.state_slots, H, self.dim, self.vdim, decay=self.decay,
                                     max_q_len=batch.max_q_len, positive_decay=min(self.decay_values) > 0)
         mixed = torch.empty((x.shape[0], vw), dtype=x.dtype, device=x.device)

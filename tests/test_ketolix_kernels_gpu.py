@@ -172,6 +172,13 @@ def test_gates_of_heads_and_of_elements():
         k.gated_norm(gpu(x), gpu(w), gpu(gate), 1e-5, out, group=group, scale=0.5)
         unit = plain.rms_unit(x.reshape(5, -1, group or 90), 1e-5).reshape(5, 90)
         np.testing.assert_allclose(out.cpu().numpy()[:, :90], unit * w * plain.sigmoid(gate) * 0.5, atol=2e-5, rtol=2e-5)
+    # wide groups (a block each): in registers up to 2,048 elements, read twice beyond
+    wide, gains, gates = rng.normal(0, 3, (3, 5200)), rng.normal(1, 0.2, 5200), rng.normal(0, 2, (3, 5200))
+    for group in (None, 2600, 1300, 650, 260):
+        out = torch.zeros((3, 5200), dtype=torch.bfloat16).cuda()
+        k.gated_norm(gpu(wide), gpu(gains), gpu(gates), 1e-5, out, group=group, scale=0.5)
+        unit = plain.rms_unit(wide.reshape(3, -1, group or 5200), 1e-5).reshape(3, 5200)
+        np.testing.assert_allclose(out.float().cpu().numpy(), unit * gains * plain.sigmoid(gates) * 0.5, atol=2e-2, rtol=2e-2)
     out = torch.zeros((5, 90)).cuda()
     k.gated_norm(gpu(x), None, None, 1e-5, out, group=45)
     np.testing.assert_allclose(out.cpu().numpy(), plain.rms_unit(x.reshape(5, 2, 45), 1e-5).reshape(5, 90), atol=2e-5, rtol=2e-5)
