@@ -21,7 +21,7 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 
 // A block per row. Queries [n_heads * dim] and keys [n_kv_heads * dim] are each RMS-normed over the WHOLE projection (all
 // heads at once) with a gain vector of that length (null: the projection goes on as it is), then the first rot_dims
-// elements of every head are rotated, element 2i with element 2i+1, by position * frequencies[i]. Queries go to q_out
+// elements of every head are rotated, element 2i with element 2i+1, by position * frequencies[i] (64-bit). Queries go to q_out
 // [rows, n_heads * head_size]; keys to the key pages; values [n_kv_heads * vdim], blended with another layer's values of
 // the same row where v_other is given (v <- (1 - mix) v + mix v_other, mix read from the device), to the value pages. The
 // pages' heads hold head_size >= dim, vdim elements, zeros beyond a head's own. A negative slot stores nothing.
@@ -29,7 +29,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void projection_rows_kernel(const float* __restrict__ q, int q_stride, const float* __restrict__ k, int k_stride,
                                                               const float* __restrict__ v, int v_stride, const float* __restrict__ v_other,
                                                               int v_other_stride, const float* __restrict__ mix, const float* __restrict__ q_gain,
-                                                              const float* __restrict__ k_gain, float eps, const float* __restrict__ frequencies,
+                                                              const float* __restrict__ k_gain, float eps, const double* __restrict__ frequencies,
                                                               int rot_dims, const int* __restrict__ positions, const int* __restrict__ slots,
                                                               T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages, int n_heads,
                                                               int n_kv_heads, int dim, int vdim, int head_size, int page_size, int write_cache) {
@@ -61,15 +61,19 @@ __global__ __launch_bounds__(256) void projection_rows_kernel(const float* __res
     }
     const float q_factor = q_gain ? 1.0f / sqrtf(q_squares / (float)q_width + eps) : 1.0f;
     const float k_factor = k_gain ? 1.0f / sqrtf(k_squares / (float)k_width + eps) : 1.0f;
-    const float position = (float)position_of_row;
+    const double position = (double)position_of_row;
     // a pair of neighbouring elements of a normed head, rotated where it lies among the first rot_dims: d its first element's place
     // in the head (even), `at` the head's first element in the row; elements beyond the head's own are zero
     auto turned_pair = [&](const float* in, const float* gain, float factor, int at, int d, float& first, float& second) {
         first = d < dim ? in[at + d] * factor * (gain ? gain[at + d] : 1.0f) : 0.0f;
         second = d + 1 < dim ? in[at + d + 1] * factor * (gain ? gain[at + d + 1] : 1.0f) : 0.0f;
         if (d < rot_dims) {
+            // the angle in 64-bit (a 32-bit product of a position in the thousands is good to 1e-4 only), brought into -pi .. pi,
+            // where its sine and cosine are taken in 32-bit
+            const double angle = position * frequencies[d >> 1];
+            const double turns = rint(angle * 0.15915494309189535);
             float s, c;
-            sincosf(position * frequencies[d >> 1], &s, &c);
+            sincosf((float)(angle - turns * 6.283185307179586), &s, &c);
             const float u = first, w = second;
             first = u * c - w * s;
             second = w * c + u * s;
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(256) void short_conv_keep_kernel(const float* __res
 
 MLLM_API int mllm_projection_rows(const float* q, int q_stride, const float* k, int k_stride, const float* v, int v_stride, const float* v_other,
                                   int v_other_stride, const float* mix, const float* q_gain, const float* k_gain, float eps,
-                                  const float* frequencies, int rot_dims, const int* positions, const int* slots, void* q_out, void* k_pages,
+                                  const double* frequencies, int rot_dims, const int* positions, const int* slots, void* q_out, void* k_pages,
                                   void* v_pages, int n_rows, int n_heads, int n_kv_heads, int dim, int vdim, int head_size, int page_size,
                                   int write_cache, int dtype, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && n_kv_heads > 0 && dim > 0 && vdim > 0 && page_size > 0, "projection_rows: bad sizes");

@@ -102,9 +102,9 @@ __global__ __launch_bounds__(512) void recurrence_kernel(const float* __restrict
                 for (int t = 0; t < n_valid; t++) {
                     const float it = __shfl(gi, t, WAVE), ft = __shfl(gf, t, WAVE);
                     const float m_new = fmaxf(ft + m, it);
-                    if (tid == 0) {
-                        keep[t] = expf(ft + m - m_new);
-                        take[t] = expf(it - m_new);
+                    if (tid == 0) {   // the differences in 64-bit: next to a large m, f + m - m' would lose what f holds
+                        keep[t] = expf((float)((double)ft + (double)m - (double)m_new));
+                        take[t] = expf((float)((double)it - (double)m_new));
                         floor_[t] = expf(-m_new);
                     }
                     m = m_new;
@@ -435,8 +435,8 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const int* __restrict__
         float keep, take, m_new = 0.0f;
         if (MODE == GATED) {
             m_new = fmaxf(total + m, mu);
-            keep = expf(total + m - m_new);
-            take = expf(mu - m_new);
+            keep = expf((float)((double)total + (double)m - (double)m_new));
+            take = expf((float)((double)mu - (double)m_new));
         } else {
             keep = expf(total);
             take = 1.0f;

@@ -1023,7 +1023,7 @@ def projection_rows(q, k, v, q_gain, k_gain, eps, frequencies, rot_dims, positio
     """The row-wise work between a mixer's projections and its attention. q [rows, n_heads * dim], k [rows, n_kv_heads * dim], v
     [rows, n_kv_heads * vdim]: float32 views whose rows may be strided (parts of a fused product). Queries and keys are RMS-normed
     over the whole projection with gain vectors of that length (None: no norm), then the first ``rot_dims`` elements of every head
-    rotated, element 2i with 2i + 1, by position * frequencies[i]. Returns q as [rows, n_heads * head_size] in the pages' type; keys
+    rotated, element 2i with 2i + 1, by position * frequencies[i] (float64 [rot_dims / 2]; the angle is taken in 64-bit). Returns q as [rows, n_heads * head_size] in the pages' type; keys
     and values go to slots[row] of the pages ([num_pages, n_kv_heads, page_size, head_size], zeros beyond dim / vdim), the values
     blended first where ``v_other`` (rows like v) and ``mix`` (a float32 number on the device) are given: (1 - mix) v + mix v_other."""
     num_pages, n_kv, page_size, head_size = k_pages.shape
@@ -1039,7 +1039,7 @@ def projection_rows(q, k, v, q_gain, k_gain, eps, frequencies, rot_dims, positio
             _device_tensor(gain, name, torch.float32, 1)
             _require(gain.shape[0] == width, f"{name} does not match the projection")
     if rot_dims:
-        _device_tensor(frequencies, "frequencies", torch.float32, 1)
+        _device_tensor(frequencies, "frequencies", torch.float64, 1)
         _require(rot_dims % 2 == 0 and rot_dims <= dim and frequencies.shape[0] >= rot_dims // 2, "the rotation does not fit the heads")
     if v_other is not None:
         _rows_f32(v_other, "v_other", n_kv_heads * vdim)

@@ -77,7 +77,7 @@ class RotaryEncoding(PositionEncoding):
                     values[i] = (1.0 - s) * f / factor + s * f
         elif self.scaling:
             raise ValueError(f"unknown kind of scaling {kind!r}: yarn or wavelength")
-        self.values = values   # float64 on the host; ``frequencies`` rounds them to 32-bit on the device
+        self.values = values   # float64 on the host; ``frequencies`` rounds them to 32-bit on the device, ``frequencies64`` does not
         self._on_device = {}
 
     def frequencies(self, device):
@@ -86,6 +86,15 @@ class RotaryEncoding(PositionEncoding):
         key = str(device)
         if key not in self._on_device:
             self._on_device[key] = torch.tensor(self.values or [0.0], dtype=torch.float64).to(torch.float32).to(device)
+        return self._on_device[key]
+
+    def frequencies64(self, device):
+        """The same numbers unrounded, for a kernel that takes its angles in 64-bit."""
+        import torch
+
+        key = (str(device), 64)
+        if key not in self._on_device:
+            self._on_device[key] = torch.tensor(self.values or [0.0], dtype=torch.float64).to(device)
         return self._on_device[key]
 
 

@@ -139,7 +139,7 @@ class ProjectionNormAttention(Mixer):
                 if v_other is None:
                     raise ValueError(f"no earlier layer of this step has left the values of group {self.value_mix!r}")
         rotary = self.rotary
-        q = kernels.projection_rows(q, k, v, self.q_norm, self.k_norm, self.eps, None if rotary is None else rotary.frequencies(x.device),
+        q = kernels.projection_rows(q, k, v, self.q_norm, self.k_norm, self.eps, None if rotary is None else rotary.frequencies64(x.device),
                                     0 if rotary is None else rotary.dims, batch.positions, ctx.group.slots, ctx.k_pages, ctx.v_pages,
                                     self.n_heads, self.n_kv_heads, self.dim, self.vdim, v_other=v_other, mix=self.vmix, write_cache=ctx.write_cache)
         mixed = kernels.paged_attention(
