@@ -377,7 +377,7 @@ def ketolix_shape(width: int, layers: int, vocab: int = 50257) -> dict:
     64 x 128 with decays from 0.9 to 0.999); feed-forwards of 8/3 x width."""
     heads, wide_heads = width // 64, max(1, width // 128)
     ff = -(-(8 * width // 3) // 64) * 64
-    rot = {"dims": 64, "base": 50000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}}
+    rot = {"dims": 64, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}}
     mlp = {"kind": "dense", "ff": ff}
     attention = {"type": "attention", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "softcap": 30.0,
                                                            "mask": {"size": 512}, "rot": rot, "v_mix": True}}
@@ -385,7 +385,7 @@ def ketolix_shape(width: int, layers: int, vocab: int = 50257) -> dict:
     decays = [1.0 - 0.1 ** (1.0 + 2.0 * i / max(1, wide_heads - 1)) for i in range(wide_heads)]
     parallel = {"type": "parallel", "mlp": mlp, "mixer": {
         "left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "conv": 4, "mask": {"size": 512},
-                 "rot": {"dims": 32, "base": 50000.0}},
+                 "rot": {"dims": 32, "base": 500000.0}},
         "right": {"heads": wide_heads, "dim": 64, "vdim": 128, "decay": decays}, "left_scale": 0.7, "right_scale": 0.7}}
     pattern = [memory, attention, attention, parallel]
     return {"architecture": "Ketolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": [pattern[i % 4] for i in range(layers)]}
