@@ -76,4 +76,14 @@ CASES = {
         parallel_layer(heads=2, kv_heads=1, dim=32, conv=5, window=64, rotation=rot(16, 300.0), right_heads=2, right_dim=16, right_vdim=130,
                        decay=(0.8, 0.99)),
     ], width=96, vocab=130),
+    # heads of 80 to 128 (pages of 96 and 128 elements a head: other attention kernels than heads of 64 take), matrices of 96 x 128
+    # and 128 x 96 (chunks of 32 rows), no softcap beside a softcap, a convolution of three taps on heads of 96
+    "large": model([
+        attention_layer(heads=4, kv_heads=2, dim=80, vdim=96, scale=80 ** -0.5, softcap=25.0, window=100, rotation=rot(40, 20000.0, (8.0, 1.0, 4.0, 64)), v_mix=True),
+        mlstm_layer(heads=2, dim=96, vdim=128, cap=10.0, ff=None),
+        attention_layer(heads=2, kv_heads=1, dim=128, vdim=192, scale=128 ** -0.5, softcap=None, window=None, rotation=rot(128, 300.0), v_mix=True, ff=None),
+        parallel_layer(heads=2, kv_heads=2, dim=96, scale=96 ** -0.5, conv=3, window=72, rotation=rot(24, 5000.0), right_heads=2, right_dim=64, right_vdim=32,
+                       decay=(0.9, 0.99), ff=200),
+        mlstm_layer(heads=1, dim=128, vdim=96, cap=None, ff=None),
+    ], width=160, vocab=211),
 }

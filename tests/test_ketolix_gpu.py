@@ -47,7 +47,7 @@ def plain_logits(config, weights, requests, bf16):
     return {name: plain.forward(config, w, tokens, round_to=plain_gpt2.stored_as_bf16 if bf16 else None) for name, tokens in requests.items()}
 
 
-LENGTHS = {"mixed": [5, 130, 64, 65, 1, 200, 33], "odd": [67, 2, 130, 31], "wide": [3, 150, 64, 17, 129]}
+LENGTHS = {"mixed": [5, 130, 64, 65, 1, 200, 33], "odd": [67, 2, 130, 31], "wide": [3, 150, 64, 17, 129], "large": [150, 70, 3, 97]}
 MODES = {"whole": replay.whole, "tail": replay.prefill_then_decode, "chunked": replay.chunked, "mixed": replay.mixed}
 # logits up to 60; sums in another order than numpy's, angles in 32-bit, and positions at which a matrix memory's normaliser
 # passes close to zero, which multiply every rounding before them
