@@ -1,5 +1,6 @@
 // Mixers that keep a matrix per head and request instead of keys and values: S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t.
-// Two kinds share one kernel:
+// Two kinds share the kernels of this file (one that walks a portion row by row, for decoding and short portions, and three
+// further down that take long portions chunk by chunk):
 //   GATED (the matrix memory of an mLSTM): log gates i_t and f_t per head and token, a running maximum m that starts at 0,
 //     m_t = max(f_t + m_(t-1), i_t), a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t); a vector n that follows the same
 //     recurrence with k alone; o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6). The gates arrive as the sums of their
@@ -8,7 +9,7 @@
 // State, gates, sums and outputs are 32-bit. The state of a request lies in its slot: S [heads, dim, vdim], then (GATED)
 // n [heads, dim] and m [heads].
 //
-// A block takes one (request, head, tile of VT value columns) and walks the request's rows of this step in order. Thread
+// Row by row: a block takes one (request, head, tile of VT value columns) and walks the request's rows of this step in order. Thread
 // (part p, column j) keeps S[p R .. p R + R - 1, j] in registers across all rows. Rows are taken TB at a time: their q, k, v
 // are staged in LDS while the first wave settles the gates of those rows (the scalar recurrence of m), then every thread
 // moves its piece of S on row by row and leaves its share of each row's output, which are added up over the parts at the end.
@@ -30,7 +31,7 @@ __global__ __launch_bounds__(512) void recurrence_kernel(const float* __restrict
                                                          const int* __restrict__ q_starts, const int* __restrict__ state_slots,
                                                          float* __restrict__ out, int out_stride, int dim, int vdim, int P, int VT, int TB) {
     extern __shared__ float lds[];
-    const int request = blockIdx.x, head = blockIdx.y, n_heads = gridDim.y;
+    const int request = blockIdx.x, head = blockIdx.y;
     const int slot = state_slots[request];
     const int first_row = q_starts[request], rows = q_starts[request + 1] - first_row;
     if (slot < 0 || rows <= 0) return;   // the whole block: a padding request, or one that brings nothing
@@ -158,7 +159,6 @@ __global__ __launch_bounds__(512) void recurrence_kernel(const float* __restrict
         if (MODE == GATED && works && jt == 0 && blockIdx.z == 0 && i0 + r < dim) mine[n_at + (size_t)head * dim + i0 + r] = n[r];
     }
     if (MODE == GATED && tid == 0 && blockIdx.z == 0) mine[m_at + head] = m;
-    (void)n_heads;
 }
 
 struct Plan {
@@ -402,59 +402,50 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const int* __restrict__
     if (MODE == GATED && first_block && tid < dim) n = mine[n_at + (size_t)head * dim + tid];
     float m = MODE == GATED ? mine[m_at + head] : 0.0f;
     auto record_of = [&](int c) { return scratch + (chunk_record(first_row + c * chunk_rows, chunk_rows, request) * n_heads + head) * record_floats; };
-    // the next chunk's numbers are asked for before this chunk's are used
-    float next[PER], next_n = 0.0f, next_total, next_mu;
-    {
-        float* record = record_of(0);
+    // the numbers of four chunks are asked for at once (a pass over the chunks one by one waits for memory at every chunk)
+    constexpr int AHEAD = 4;
+    for (int c0 = 0; c0 < n_chunks; c0 += AHEAD) {
+        float sums[AHEAD][PER], sum_n[AHEAD], total[AHEAD], mu[AHEAD];
 #pragma unroll
-        for (int u = 0; u < PER; u++) {
-            const size_t e = base + (size_t)u * 256 + tid;
-            next[u] = e < elements ? record[e] : 0.0f;
-        }
-        if (MODE == GATED && first_block && tid < dim) next_n = record[elements + tid];
-        next_total = record[record_floats - 4];
-        next_mu = record[record_floats - 3];
-    }
-    for (int c = 0; c < n_chunks; c++) {
-        float* record = record_of(c);
-        float sums[PER];
-#pragma unroll
-        for (int u = 0; u < PER; u++) sums[u] = next[u];
-        const float sum_n = next_n, total = next_total, mu = next_mu;
-        if (c + 1 < n_chunks) {
-            float* ahead = record_of(c + 1);
+        for (int d = 0; d < AHEAD; d++) {
+            const float* record = record_of(min(c0 + d, n_chunks - 1));
 #pragma unroll
             for (int u = 0; u < PER; u++) {
                 const size_t e = base + (size_t)u * 256 + tid;
-                next[u] = e < elements ? ahead[e] : 0.0f;
+                sums[d][u] = record[min(e, elements - 1)];
             }
-            if (MODE == GATED && first_block && tid < dim) next_n = ahead[elements + tid];
-            next_total = ahead[record_floats - 4];
-            next_mu = ahead[record_floats - 3];
-        }
-        float keep, take, m_new = 0.0f;
-        if (MODE == GATED) {
-            m_new = fmaxf(total + m, mu);
-            keep = expf((float)((double)total + (double)m - (double)m_new));
-            take = expf((float)((double)mu - (double)m_new));
-        } else {
-            keep = expf(total);
-            take = 1.0f;
+            sum_n[d] = MODE == GATED && first_block ? record[elements + min(tid, dim - 1)] : 0.0f;
+            total[d] = record[record_floats - 4];
+            mu[d] = record[record_floats - 3];
         }
 #pragma unroll
-        for (int u = 0; u < PER; u++) {
-            const size_t e = base + (size_t)u * 256 + tid;
-            if (e < elements) record[e] = S[u];
-            S[u] = keep * S[u] + take * sums[u];
-        }
-        if (MODE == GATED && first_block) {
-            if (tid < dim) {
-                record[elements + tid] = n;
-                n = keep * n + take * sum_n;
+        for (int d = 0; d < AHEAD; d++) {
+            if (c0 + d >= n_chunks) break;
+            float* record = record_of(c0 + d);
+            float keep, take, m_new = 0.0f;
+            if (MODE == GATED) {
+                m_new = fmaxf(total[d] + m, mu[d]);
+                keep = expf((float)((double)total[d] + (double)m - (double)m_new));
+                take = expf((float)((double)mu[d] - (double)m_new));
+            } else {
+                keep = expf(total[d]);
+                take = 1.0f;
             }
-            if (tid == 0) record[record_floats - 2] = m;
+#pragma unroll
+            for (int u = 0; u < PER; u++) {
+                const size_t e = base + (size_t)u * 256 + tid;
+                if (e < elements) record[e] = S[u];
+                S[u] = keep * S[u] + take * sums[d][u];
+            }
+            if (MODE == GATED && first_block) {
+                if (tid < dim) {
+                    record[elements + tid] = n;
+                    n = keep * n + take * sum_n[d];
+                }
+                if (tid == 0) record[record_floats - 2] = m;
+            }
+            m = m_new;
         }
-        m = m_new;
     }
 #pragma unroll
     for (int u = 0; u < PER; u++) {
@@ -590,6 +581,220 @@ __global__ __launch_bounds__(CHUNK_THREADS) void chunk_output_kernel(const float
     }
 }
 
+// The same two kernels for chunks of 64 rows (heads up to 64 wide) with their products on the matrix cores, in 32-bit
+// (v_mfma_f32_32x32x2_f32: the first operand's lane holds row l % 32 and k = l / 32, the second's column l % 32 and k = l / 32; a
+// lane's sixteen sums are rows 8 (v / 4) + 4 (l / 32) + v % 4 of column l % 32). Operands lie in LDS so that a lane's row or column
+// is a lane's bank: q and k transposed ([i][t], rows of 65), v and the weighted keys as they come.
+constexpr int CHUNK_PAD = 65;
+
+template <int MODE>
+__global__ __launch_bounds__(CHUNK_THREADS) void chunk_sums_mfma_kernel(const float* __restrict__ k, int k_stride, const float* __restrict__ v, int v_stride,
+                                                                        const float* __restrict__ gate_in, const float* __restrict__ gate_forget,
+                                                                        int gate_stride, float cap, const float* __restrict__ decay,
+                                                                        const int* __restrict__ q_starts, const int* __restrict__ state_slots,
+                                                                        float* __restrict__ scratch, int dim, int vdim, int tiles) {
+    constexpr int L = 64;
+    __shared__ float Ks[L][64];          // [s][i], already times the row's weight
+    __shared__ float Vs[L][CHUNK_VT];
+    __shared__ float weight[L];
+    const int request = blockIdx.x, head = blockIdx.y, n_heads = gridDim.y, chunk = blockIdx.z / tiles, tile = blockIdx.z % tiles;
+    const int first_row = q_starts[request], rows = q_starts[request + 1] - first_row;
+    if (state_slots[request] < 0 || chunk * L >= rows) return;
+    const int n_valid = min(L, rows - chunk * L), chunk_first = first_row + chunk * L;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const size_t record_floats = (size_t)dim * vdim + dim + 4;
+    float* record = scratch + (chunk_record(chunk_first, L, request) * n_heads + head) * record_floats;
+
+    // a thread's eight elements of k and of v (column tid % 64 of rows tid / 64 + 8 u) are asked for at once, from clamped places,
+    // before the first wave settles the gates: one wait for memory
+    constexpr int PER = L * 64 / CHUNK_THREADS;
+    const int my_column = tid % 64, my_row = tid / 64;
+    float k_mine[PER], v_mine[PER];
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const size_t row = (size_t)(chunk_first + min(my_row + u * (CHUNK_THREADS / 64), n_valid - 1));
+        k_mine[u] = k[row * k_stride + head * dim + min(my_column, dim - 1)];
+        v_mine[u] = v[row * v_stride + head * vdim + min(tile * CHUNK_VT + my_column, vdim - 1)];
+    }
+    if (wave == 0) {
+        float log_keep = 0.0f, log_take = 0.0f;
+        if (lane < n_valid) row_gates<MODE>(gate_in, gate_forget, gate_stride, cap, MODE == DECAYED ? logf(decay[head]) : 0.0f, (size_t)(chunk_first + lane), head, log_keep, log_take);
+        const double b = lanes_prefix_sum((double)log_keep, lane);
+        const double total = __shfl(b, n_valid - 1, WAVE);
+        const double reach = lane < n_valid ? (total - b) + (double)log_take : -INFINITY;
+        const float mu = MODE == GATED ? wave_max((float)reach) : 0.0f;
+        weight[lane] = lane < n_valid ? expf((float)(reach - (double)mu)) : 0.0f;
+        if (lane == 0 && tile == 0) {
+            record[record_floats - 4] = (float)total;
+            record[record_floats - 3] = mu;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const int s = my_row + u * (CHUNK_THREADS / 64);
+        float kv = k_mine[u], vv = v_mine[u];
+        if (MODE == DECAYED) kv = silu_f(kv), vv = silu_f(vv);
+        Ks[s][my_column] = s < n_valid && my_column < dim ? kv * weight[s] : 0.0f;
+        Vs[s][my_column] = s < n_valid && tile * CHUNK_VT + my_column < vdim ? vv : 0.0f;
+    }
+    __syncthreads();
+    const int half = lane / 32, l32 = lane % 32;
+    if (wave < 4 && (wave / 2) * 32 < dim) {   // U = (weighted K)^T V: a wave a tile of 32 rows i x 32 columns j
+        const int ib = wave / 2, jb = wave % 2;
+        f32x16 acc;
+#pragma unroll
+        for (int u = 0; u < 16; u++) acc[u] = 0.0f;
+        const int s_end = (n_valid + 1) & ~1;
+        for (int s = 0; s < s_end; s += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Ks[s + half][ib * 32 + l32], Vs[s + half][jb * 32 + l32], acc, 0, 0, 0);
+        const int j = tile * CHUNK_VT + jb * 32 + l32;
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int i = ib * 32 + 8 * (u / 4) + 4 * half + (u % 4);
+            if (i < dim && j < vdim) record[(size_t)i * vdim + j] = acc[u];
+        }
+    }
+    if (MODE == GATED && tile == 0 && wave >= 4 && tid - 4 * WAVE < dim) {   // the chunk's share of n
+        const int i = tid - 4 * WAVE;
+        float sum = 0.0f;
+        for (int s = 0; s < n_valid; s++) sum += Ks[s][i];
+        record[(size_t)dim * vdim + i] = sum;
+    }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(CHUNK_THREADS) void chunk_output_mfma_kernel(const float* __restrict__ q, int q_stride, const float* __restrict__ k, int k_stride,
+                                                                          const float* __restrict__ v, int v_stride, const float* __restrict__ gate_in,
+                                                                          const float* __restrict__ gate_forget, int gate_stride, float cap,
+                                                                          const float* __restrict__ decay, float q_scale, const int* __restrict__ q_starts,
+                                                                          const int* __restrict__ state_slots, const float* __restrict__ scratch,
+                                                                          float* __restrict__ out, int out_stride, int dim, int vdim, int tiles) {
+    constexpr int L = 64, PAD = CHUNK_PAD;
+    __shared__ float Qt[64 * PAD];        // [i][t]; behind the products: the outputs [t][j]
+    __shared__ float Kt[64 * PAD];        // [i][s]; behind the scores: the weighted scores [s][t]
+    __shared__ float Vs[L][CHUNK_VT];     // [s][j]
+    __shared__ double b_of[L];
+    __shared__ double m_of[L];
+    __shared__ float take_of[L], start_weight[L], nq_inside[2][L], nq_before[L];
+    const int request = blockIdx.x, head = blockIdx.y, n_heads = gridDim.y, chunk = blockIdx.z / tiles, tile = blockIdx.z % tiles;
+    const int first_row = q_starts[request], rows = q_starts[request + 1] - first_row;
+    if (state_slots[request] < 0 || chunk * L >= rows) return;
+    const int n_valid = min(L, rows - chunk * L), chunk_first = first_row + chunk * L;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int half = lane / 32, l32 = lane % 32;
+    const size_t elements = (size_t)dim * vdim, record_floats = elements + dim + 4;
+    const float* record = scratch + (chunk_record(chunk_first, L, request) * n_heads + head) * record_floats;
+
+    {   // a thread's eight elements of q, k and v (column tid % 64 of rows tid / 64 + 8 u), asked for at once from clamped places
+        constexpr int PER = L * 64 / CHUNK_THREADS;
+        const int my_column = tid % 64, my_row = tid / 64;
+        float q_mine[PER], k_mine[PER], v_mine[PER];
+#pragma unroll
+        for (int u = 0; u < PER; u++) {
+            const size_t row = (size_t)(chunk_first + min(my_row + u * (CHUNK_THREADS / 64), n_valid - 1));
+            q_mine[u] = q[row * q_stride + head * dim + min(my_column, dim - 1)];
+            k_mine[u] = k[row * k_stride + head * dim + min(my_column, dim - 1)];
+            v_mine[u] = v[row * v_stride + head * vdim + min(tile * CHUNK_VT + my_column, vdim - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < PER; u++) {
+            const int s = my_row + u * (CHUNK_THREADS / 64);
+            float qv = q_mine[u], kv = k_mine[u], vv = v_mine[u];
+            if (MODE == DECAYED) qv = silu_f(qv), kv = silu_f(kv), vv = silu_f(vv);
+            const bool row_counts = s < n_valid;
+            if (my_column < dim) {
+                Qt[my_column * PAD + s] = row_counts ? qv * q_scale : 0.0f;
+                Kt[my_column * PAD + s] = row_counts ? kv : 0.0f;
+            }
+            Vs[s][my_column] = row_counts && tile * CHUNK_VT + my_column < vdim ? vv : 0.0f;
+        }
+    }
+    if (wave == 0) {
+        float log_keep = 0.0f, log_take = 0.0f;
+        if (lane < n_valid) row_gates<MODE>(gate_in, gate_forget, gate_stride, cap, MODE == DECAYED ? logf(decay[head]) : 0.0f, (size_t)(chunk_first + lane), head, log_keep, log_take);
+        const double b = lanes_prefix_sum((double)log_keep, lane);
+        double m_row = 0.0, from_start = b;
+        if (MODE == GATED) {
+            const double m_start = (double)record[record_floats - 2];
+            const double best = lanes_prefix_max(lane < n_valid ? (double)log_take - b : -INFINITY, lane);
+            m_row = b + fmax(m_start, best);
+            from_start = b + m_start - m_row;
+        }
+        b_of[lane] = b;
+        m_of[lane] = m_row;
+        take_of[lane] = log_take;
+        start_weight[lane] = expf((float)from_start);
+    }
+    __syncthreads();
+    // ---- scores, transposed: rows the keys s, columns the queries t; the three tiles that hold a visible pair, a wave each ----
+    f32x16 acc;
+#pragma unroll
+    for (int u = 0; u < 16; u++) acc[u] = 0.0f;
+    const int key_block = wave == 2 ? 1 : 0, query_block = wave == 0 ? 0 : 1;
+    if (wave < 3) {
+        for (int i = 0; i < dim; i += 2)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[(i + half) * PAD + key_block * 32 + l32], Qt[(i + half) * PAD + query_block * 32 + l32], acc, 0, 0, 0);
+        const int t = query_block * 32 + l32;
+        float column_sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int s = key_block * 32 + 8 * (u / 4) + 4 * half + (u % 4);
+            const bool sees = s <= t && t < n_valid;
+            acc[u] = sees ? acc[u] * expf((float)((b_of[t] - b_of[s]) + (double)take_of[s] - m_of[t])) : 0.0f;
+            column_sum += acc[u];
+        }
+        column_sum += __shfl_xor(column_sum, 32, WAVE);
+        if (half == 0) nq_inside[key_block][t] = column_sum;
+    } else if (wave == 3) {
+        if (lane < 32) nq_inside[1][lane] = 0.0f;   // no key of the second block is seen by a query of the first
+    } else if (wave == 4 && MODE == GATED) {
+        const float* n_start = record + elements;
+        float sum = 0.0f;
+        for (int i = 0; i < dim; i++) sum += Qt[i * PAD + lane] * n_start[i];
+        nq_before[lane] = sum;
+    }
+    __syncthreads();   // everybody has read the keys
+    float* At = Kt;    // [s][t]
+    if (wave < 3) {
+#pragma unroll
+        for (int u = 0; u < 16; u++) At[(key_block * 32 + 8 * (u / 4) + 4 * half + (u % 4)) * PAD + query_block * 32 + l32] = acc[u];
+    } else if (wave == 3) {
+#pragma unroll
+        for (int u = 0; u < 16; u++) At[(32 + 8 * (u / 4) + 4 * half + (u % 4)) * PAD + l32] = 0.0f;
+    }
+    __syncthreads();
+    // ---- outputs, transposed: rows the tile's columns j, columns the queries t; four tiles, a wave each ----
+    float value[16];
+    const int j_block = wave / 2, t_block = wave % 2;
+    if (wave < 4) {
+        f32x16 inside, before;
+#pragma unroll
+        for (int u = 0; u < 16; u++) inside[u] = before[u] = 0.0f;
+        const int s_end = min(t_block == 0 ? 32 : 64, (n_valid + 1) & ~1);
+        for (int s = 0; s < s_end; s += 2)
+            inside = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[s + half][j_block * 32 + l32], At[(s + half) * PAD + t_block * 32 + l32], inside, 0, 0, 0);
+        const int column = min(tile * CHUNK_VT + j_block * 32 + l32, vdim - 1);
+        for (int i = 0; i < dim; i += 2)
+            before = __builtin_amdgcn_mfma_f32_32x32x2f32(record[(size_t)(i + half) * vdim + column], Qt[(i + half) * PAD + t_block * 32 + l32], before, 0, 0, 0);
+        const int t = t_block * 32 + l32;
+        float divide = 1.0f;
+        if (MODE == GATED) divide = 1.0f / (fmaxf(fabsf(nq_inside[0][t] + nq_inside[1][t] + start_weight[t] * nq_before[t]), expf((float)-m_of[t])) + 1e-6f);
+#pragma unroll
+        for (int u = 0; u < 16; u++) value[u] = (inside[u] + start_weight[t] * before[u]) * divide;
+    }
+    __syncthreads();   // everybody has read the queries
+    float* Ot = Qt;    // [t][j]
+    if (wave < 4) {
+#pragma unroll
+        for (int u = 0; u < 16; u++) Ot[(t_block * 32 + l32) * PAD + j_block * 32 + 8 * (u / 4) + 4 * half + (u % 4)] = value[u];
+    }
+    __syncthreads();
+    for (int e = tid; e < n_valid * CHUNK_VT; e += CHUNK_THREADS) {
+        const int t = e / CHUNK_VT, j = tile * CHUNK_VT + e % CHUNK_VT;
+        if (j < vdim) out[(size_t)(chunk_first + t) * out_stride + head * vdim + j] = Ot[t * PAD + e % CHUNK_VT];
+    }
+}
+
 int chunk_rows_for(int dim) { return dim <= 64 ? 64 : (dim <= 128 ? 32 : 16); }
 
 }  // namespace
@@ -633,15 +838,27 @@ MLLM_API int mllm_recurrence_chunked(int kind, const float* q, int q_stride, con
         chunk_output_kernel<LL, MODE><<<grid, CHUNK_THREADS, 0, stream>>>(q, q_stride, k, k_stride, v, v_stride, gate_in, gate_forget, gate_stride, cap, \
                                                                           decay, q_scale, q_starts, state_slots, scratch, out, out_stride, dim, vdim, tiles); \
     } while (0)
+#define CHUNKED_MFMA(MODE)                                                                                                                         \
+    do {                                                                                                                                           \
+        mllm_count_kernel(MLLM_K_RECURRENCE);                                                                                                      \
+        chunk_sums_mfma_kernel<MODE><<<grid, CHUNK_THREADS, 0, stream>>>(k, k_stride, v, v_stride, gate_in, gate_forget, gate_stride, cap, decay, q_starts, \
+                                                                         state_slots, scratch, dim, vdim, tiles);                                  \
+        mllm_count_kernel(MLLM_K_RECURRENCE);                                                                                                      \
+        chunk_scan_kernel<MODE><<<scan_grid, 256, 0, stream>>>(q_starts, state_slots, scratch, state, state_stride, n_at, m_at, dim, vdim, 64);      \
+        mllm_count_kernel(MLLM_K_RECURRENCE);                                                                                                      \
+        chunk_output_mfma_kernel<MODE><<<grid, CHUNK_THREADS, 0, stream>>>(q, q_stride, k, k_stride, v, v_stride, gate_in, gate_forget, gate_stride, cap, \
+                                                                           decay, q_scale, q_starts, state_slots, scratch, out, out_stride, dim, vdim, tiles); \
+    } while (0)
     if (kind == GATED) {
-        if (L == 64) CHUNKED(64, GATED);
+        if (L == 64) CHUNKED_MFMA(GATED);
         else if (L == 32) CHUNKED(32, GATED);
         else CHUNKED(16, GATED);
     } else {
-        if (L == 64) CHUNKED(64, DECAYED);
+        if (L == 64) CHUNKED_MFMA(DECAYED);
         else if (L == 32) CHUNKED(32, DECAYED);
         else CHUNKED(16, DECAYED);
     }
+#undef CHUNKED_MFMA
 #undef CHUNKED
     return mllm_check_launch("recurrence_chunked");
 }
